@@ -1,0 +1,84 @@
+"""The Python entry point: load a model folder (or build random weights from a configuration),
+make an engine over a cache, step it, generate from it.
+
+The reference's surface this corresponds to is Llama3Model::{from_gguf, forward, generate, reset}
+(llama3.rs:12886, 13496, 16042, 13488) and the sampling functions (src/sampling.rs:10-123).
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional, Sequence, Union
+
+import torch
+
+from .config import config_from_dict, load_config
+from .engine.model import CausalLM
+from .engine.step import Engine
+from .engine.generate import GenerationResult, Generator
+from .hip import ops
+from .parts import Precision
+from .weights.loader import init_random, load_weights
+
+
+class Model:
+    def __init__(self, config, lm: CausalLM):
+        self.config = config
+        self.lm = lm
+        self.precision = lm.precision
+        self.device = lm.device
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def load(cls, folder: str, dtype=None, device: Union[str, torch.device, None] = None) -> "Model":
+        """A folder with config.json and model.safetensors; the model class is chosen by config.json."""
+        config = load_config(folder)
+        device = torch.device(device) if device is not None else ops.require_gpu()
+        precision = Precision.of(dtype or getattr(config, "torch_dtype", "bfloat16"))
+        lm = CausalLM(config.plan(), precision, device)
+        load_weights(lm, folder)
+        return cls(config, lm)
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype=None, device=None, stored_dtype: Optional[torch.dtype] = None) -> "Model":
+        """Random weights straight onto the device: the same tensors write_random_model(config, seed) writes."""
+        if isinstance(config, dict):
+            config = config_from_dict(config)
+        device = torch.device(device) if device is not None else ops.require_gpu()
+        precision = Precision.of(dtype or getattr(config, "torch_dtype", "bfloat16"))
+        lm = CausalLM(config.plan(), precision, device)
+        if stored_dtype is None:
+            stored_dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[getattr(config, "torch_dtype", "bfloat16")]
+        init_random(lm, seed, stored_dtype)
+        return cls(config, lm)
+
+    # ------------------------------------------------------------------ use
+    def engine(self, max_tokens: int, max_seqs: Optional[int] = None) -> Engine:
+        return Engine(self.lm, max_tokens=max_tokens, max_seqs=max_seqs)
+
+    new_cache = engine
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: Union[int, Sequence[int]] = 256,
+                 temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
+                 stop_token_ids: Optional[Sequence[int]] = None, max_batch: Optional[int] = None,
+                 max_tokens: Optional[int] = None, engine: Optional[Engine] = None) -> List[GenerationResult]:
+        """Generate for every prompt (token ids); as many batches one after another as needed."""
+        if prompts and isinstance(prompts[0], int):
+            prompts = [prompts]
+        caps = [max_new_tokens] * len(prompts) if isinstance(max_new_tokens, int) else list(max_new_tokens)
+        if engine is None:
+            batch = max_batch or len(prompts)
+            longest = sorted((len(p) + c for p, c in zip(prompts, caps)), reverse=True)[:batch]
+            need = sum(-(-n // 64) * 64 for n in longest)
+            engine = self.engine(max_tokens or need, max_seqs=batch)
+        if stop_token_ids is None:
+            stop_token_ids = self.lm.plan.stop_token_ids
+        gen = Generator(engine, temperature=temperature, top_k=top_k, top_p=top_p, seed=seed,
+                        stop_token_ids=stop_token_ids, max_batch=max_batch)
+        return gen.run(prompts, caps)
+
+
+def load(path_or_config, dtype=None, random_seed: Optional[int] = None, device=None) -> Model:
+    """load("folder") reads a model folder; load(config_dict_or_object, random_seed=0) makes random weights."""
+    if isinstance(path_or_config, (str, os.PathLike)):
+        return Model.load(os.fspath(path_or_config), dtype, device)
+    return Model.random(path_or_config, random_seed or 0, dtype, device)

@@ -1,0 +1,1 @@
+from .paged import Cache, CacheError, LayerCache, PageGroup, SlotTable, PAGE_SIZE

@@ -1,0 +1,70 @@
+// C interface of the HIP library (gfx950).  Every function takes raw device pointers and a HIP
+// stream, checks its arguments on the host before it launches anything, and returns 0 on success;
+// otherwise alice_last_error() describes the problem.  dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#define ALICE_ABI_VERSION 1
+
+#define ALICE_EPI_NONE 0
+#define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
+#define ALICE_EPI_SOFTCAP 2   // y = cap * tanh(y / cap)
+
+#define ALICE_LAYOUT_ROW 0     // row-major [N, K]
+#define ALICE_LAYOUT_FRAG16 1  // bfloat16 in 16x32 MFMA fragments, see linear_mfma.hip
+
+#define ALICE_LINEAR_AUTO 0
+#define ALICE_LINEAR_GENERIC 1
+#define ALICE_LINEAR_SKINNY 2
+#define ALICE_LINEAR_MFMA 3
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* alice_last_error();
+int alice_abi_version();
+int alice_device_arch(char* out, int cap);
+
+int alice_embed(const int* tokens, const void* table, int table_dtype, int table_layout, float* out,
+                int T, int H, int V, float scale, hipStream_t stream);
+
+int alice_add_norm(float* resid, const float* branch, int n_partials, long partial_stride,
+                   const void* w_post, const void* w_pre, int w_dtype, void* out, int out_dtype,
+                   const int* rows, int T, int H, float eps_post, float eps_pre, float off_post,
+                   float off_pre, int full_precision, hipStream_t stream);
+
+int alice_softcap(float* x, long n, float cap, int full_precision, hipStream_t stream);
+
+// y[M, N] = x[M, K] . W^T with an optional epilogue.  `variant` forces a kernel (tests); AUTO picks.
+// For GEGLU, W has 2N rows.  `split_k` > 1 asks for partial sums y[split_k][M][N] in float32
+// (no epilogue), to be added up by the consumer (alice_add_norm's n_partials).
+int alice_linear(const void* x, int x_dtype, const void* w, int w_dtype, int w_layout, void* y, int y_dtype,
+                 int M, int N, int K, int epilogue, float epi_param, int split_k, int variant,
+                 int full_precision, hipStream_t stream);
+// How many partial sums AUTO would like for this shape (1 = none).
+int alice_linear_split_hint(int M, int N, int K, int w_layout);
+
+// Rearranges a row-major bfloat16 [N, K] matrix into the fragment layout ([Np/16][Kp/32][64][8],
+// zero padded); dst holds Np * Kp elements with Np = ceil16(N), Kp = ceil32(K).
+int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream);
+
+int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool, void* v_pool,
+                           const float* cos_t, const float* sin_t, const int* positions,
+                           const int* seq_of_token, const int* block_table, int bt_stride, int T,
+                           int row_width, int nH, int nKV, int d, int rotary_dim, int page_size, int n_pages,
+                           hipStream_t stream);
+
+int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
+                            const int* positions, const int* seq_of_token, const int* block_table,
+                            int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
+                            float softcap, int window, int full_precision, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+
+// internal
+int alice_linear_generic(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype,
+                         int M, int N, int K, int epi, float epi_param, int full_precision,
+                         hipStream_t stream);
+#endif

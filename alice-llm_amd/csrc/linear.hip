@@ -1,0 +1,30 @@
+// Dispatch of the matrix product to its kernels.
+#include "common.h"
+#include "alice_hip.h"
+
+extern "C" int alice_linear_split_hint(int M, int N, int K, int w_layout) {
+  (void)M; (void)N; (void)K; (void)w_layout;
+  return 1;
+}
+
+extern "C" int alice_linear(const void* x, int x_dtype, const void* w, int w_dtype, int w_layout, void* y,
+                            int y_dtype, int M, int N, int K, int epilogue, float epi_param, int split_k,
+                            int variant, int full_precision, hipStream_t stream) {
+  ALICE_CHECK(x && w && y, "linear: null operand");
+  ALICE_CHECK(split_k >= 1, "linear: split_k must be at least 1");
+  if (w_layout == ALICE_LAYOUT_ROW) {
+    ALICE_CHECK(variant == ALICE_LINEAR_AUTO || variant == ALICE_LINEAR_GENERIC,
+                "linear: row-major weights run on the generic kernel only");
+    ALICE_CHECK(split_k == 1, "linear: the generic kernel produces no partial sums");
+    return alice_linear_generic(x, x_dtype, w, w_dtype, y, y_dtype, M, N, K, epilogue, epi_param,
+                                full_precision, stream);
+  }
+  alice_set_error("linear: unknown weight layout %d", w_layout);
+  return 1;
+}
+
+extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream) {
+  (void)src; (void)dst; (void)N; (void)K; (void)stream;
+  alice_set_error("to_frag16: not built");
+  return 1;
+}

@@ -1,0 +1,93 @@
+// Rotation of q and k by the position tables, and the write of k (rotated) and v into the
+// paged cache, in one pass over the fused q|k|v rows.
+//
+// Pairing is half-split over the rotated width R: (j, j + R/2), y[j] = x[j] cos - x[j+R/2] sin,
+// y[j+R/2] = x[j] sin + x[j+R/2] cos (llama3.rs:5367-5378); k is cached after the rotation and
+// v as it is (llama3.rs:14307-14331).  Dimensions at or beyond R pass through unchanged.
+#include "common.h"
+#include "alice_hip.h"
+
+// One block per token.  qkv row of row_w elements: [nH*d | nKV*d | nKV*d | ...]; with no pools
+// only the q part is read.  cos/sin: [max_pos, R/2].
+// Cache pools: [page][nKV][page_size][d]; the page of position p of sequence s is
+// block_table[s * bt_stride + p / page_size].
+template <typename T>
+__global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                                  T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                  const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                  const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                                  const int* __restrict__ block_table, int bt_stride, int row_w,
+                                  int nH, int nKV, int d, int R, int page_size, int n_pages) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = R >> 1;
+  const T* row = qkv + (size_t)t * row_w;
+  const float* cs = cos_t ? cos_t + (size_t)pos * half : nullptr;
+  const float* sn = sin_t ? sin_t + (size_t)pos * half : nullptr;
+
+  T* kdst = nullptr;
+  T* vdst = nullptr;
+  if (k_pool) {
+    const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
+    if (page >= 0 && page < n_pages) {
+      const size_t base = ((size_t)page * nKV * page_size + (size_t)(pos % page_size)) * d;
+      kdst = k_pool + base;      // head h adds h * page_size * d
+      vdst = v_pool + base;
+    }
+  }
+  const int hd2 = d >> 1;        // work items per head: one per pair of the first/second half
+  // q heads and k heads: item = (head, j) with j < d/2 handling elements j and j + d/2 when both lie
+  // in the rotated width, else copying them.
+  const int n_items = (nH + (k_pool ? nKV : 0)) * hd2;
+  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+    const int h = it / hd2, j = it % hd2;
+    const bool is_q = h < nH;
+    const T* src = row + (size_t)h * d;                     // k heads follow the q heads directly
+    T* dst;
+    if (is_q) dst = q_out + (size_t)t * nH * d + (size_t)h * d;
+    else {
+      if (!kdst) continue;
+      dst = kdst + (size_t)(h - nH) * page_size * d;
+    }
+    // Elements of this item: the rotated pair (j, j + half) if j < half, and the pass-through
+    // elements are handled by the items with j >= half: each copies e = half + j and, when
+    // R < d, nothing is lost because e ranges over [2*half .. ) below.
+    if (j < half) {
+      float x0 = load_f32(src, j), x1 = load_f32(src, j + half);
+      float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
+      store_f32(dst, j, x0 * c - x1 * s);
+      store_f32(dst, j + half, x0 * s + x1 * c);
+    }
+    // pass-through elements: indices R .. d-1, spread over the items j of this head
+    for (int e = R + j; e < d; e += hd2) store_f32(dst, e, load_f32(src, e));
+  }
+  if (vdst) {
+    const T* vsrc = row + (size_t)(nH + nKV) * d;
+    for (int it = threadIdx.x; it < nKV * d; it += blockDim.x) {
+      const int h = it / d, e = it % d;
+      vdst[(size_t)h * page_size * d + e] = vsrc[it];
+    }
+  }
+}
+
+extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool, void* v_pool,
+                                      const float* cos_t, const float* sin_t, const int* positions,
+                                      const int* seq_of_token, const int* block_table, int bt_stride,
+                                      int T, int row_width, int nH, int nKV, int d, int rotary_dim, int page_size,
+                                      int n_pages, hipStream_t stream) {
+  ALICE_CHECK(dtype_ok(dtype), "rope: unknown dtype %d", dtype);
+  ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 2 && d % 2 == 0, "rope: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
+  ALICE_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0, "rope: rotated width %d must be even and at most head_dim %d", rotary_dim, d);
+  ALICE_CHECK((cos_t == nullptr) == (sin_t == nullptr), "rope: cos and sin tables must come together");
+  ALICE_CHECK(rotary_dim == 0 || cos_t != nullptr, "rope: a rotated width needs the tables");
+  ALICE_CHECK((k_pool == nullptr) == (v_pool == nullptr), "rope: key and value pools must come together");
+  ALICE_CHECK(k_pool == nullptr || (block_table && seq_of_token && page_size > 0 && n_pages > 0 && nKV >= 1),
+              "rope: a cache write needs the block table, the token-to-sequence map and the page geometry");
+  ALICE_CHECK(row_width >= (nH + (k_pool ? 2 * nKV : 0)) * d, "rope: rows of %d elements are too short for the heads", row_width);
+  if (T == 0) return 0;
+  DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<T, 256, 0, stream>>>(
+      (const TT*)qkv, (TT*)q_out, (TT*)k_pool, (TT*)v_pool, cos_t, sin_t, positions, seq_of_token,
+      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages)));
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,306 @@
+"""Python bindings of the HIP library: one function per kernel entry point.
+
+Each wrapper checks on the host that operand shapes, dtypes and devices match what its kernel
+assumes, then calls the C function on torch's current HIP stream.  There is no other
+implementation behind these functions: without the library, or without a GPU, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional
+
+import torch
+
+from ..csrc import build as _build
+
+EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
+LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
+LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA = 0, 1, 2, 3
+ABI_VERSION = 1
+
+_lib = None
+_lock = threading.Lock()
+
+
+class HipLibraryError(RuntimeError):
+    """The HIP library is missing, cannot be built or loaded, or a kernel refused its arguments."""
+
+
+def _declare(lib) -> None:
+    c = ctypes
+    P, I, L, F = c.c_void_p, c.c_int, c.c_long, c.c_float
+    lib.alice_last_error.restype = c.c_char_p
+    lib.alice_abi_version.restype = I
+    lib.alice_device_arch.argtypes = [c.c_char_p, I]
+    sigs = {
+        "alice_embed": [P, P, I, I, P, I, I, I, F, P],
+        "alice_add_norm": [P, P, I, L, P, P, I, P, I, P, I, I, F, F, F, F, I, P],
+        "alice_softcap": [P, L, F, I, P],
+        "alice_linear": [P, I, P, I, I, P, I, I, I, I, I, F, I, I, I, P],
+        "alice_linear_split_hint": [I, I, I, I],
+        "alice_to_frag16": [P, P, I, I, P],
+        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
+        "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = I
+
+
+def library():
+    """The loaded HIP library; built with hipcc at the first call if no built one is found."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = _build.find_library()
+        if path is None:
+            try:
+                path = _build.build(verbose=True)
+            except Exception as e:
+                raise HipLibraryError(f"the HIP library is not built and building it failed: {e}") from e
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise HipLibraryError(f"cannot load {path}: {e}") from e
+        _declare(lib)
+        if lib.alice_abi_version() != ABI_VERSION:
+            raise HipLibraryError(f"{path} has interface version {lib.alice_abi_version()}, these bindings "
+                                  f"need {ABI_VERSION}: rebuild it (python -m alice_llm_amd.csrc.build)")
+        _lib = lib
+        return _lib
+
+
+def library_path() -> Optional[str]:
+    return _build.find_library()
+
+
+def require_gpu() -> torch.device:
+    if not torch.cuda.is_available():
+        raise HipLibraryError("no GPU is visible to torch: this library runs on an MI355X (gfx950) only "
+                              "and has no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _call(name: str, *args) -> None:
+    lib = library()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise HipLibraryError(f"{name}: {lib.alice_last_error().decode()}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return 0
+    if dt == torch.bfloat16:
+        return 1
+    raise HipLibraryError(f"dtype {dt} has no kernel: float32 and bfloat16 only")
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None, shape=None) -> int:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise HipLibraryError(f"{name} must be a GPU tensor")
+    if not t.is_contiguous():
+        raise HipLibraryError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise HipLibraryError(f"{name} must be {dtype}, found {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise HipLibraryError(f"{name} must have shape {tuple(shape)}, found {tuple(t.shape)}")
+    return t.data_ptr()
+
+
+def _opt(t, name, dtype=None, shape=None) -> Optional[int]:
+    return None if t is None else _dev(t, name, dtype, shape)
+
+
+# ------------------------------------------------------------------------------------ ops
+
+def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float,
+          vocab: int, dim: int, layout: int = LAYOUT_ROW) -> None:
+    T = tokens.numel()
+    _dev(tokens, "tokens", torch.int32)
+    _dev(out, "out", torch.float32, (T, dim))
+    if layout == LAYOUT_ROW:
+        _dev(table, "table", None, (vocab, dim))
+    else:
+        _dev(table, "table", torch.bfloat16)
+        need = ((vocab + 15) // 16 * 16) * ((dim + 31) // 32 * 32)
+        if table.numel() != need:
+            raise HipLibraryError(f"table in fragment layout must hold {need} elements, found {table.numel()}")
+    _call("alice_embed", tokens.data_ptr(), table.data_ptr(), dtype_code(table.dtype), layout,
+          out.data_ptr(), T, dim, vocab, float(scale), _stream())
+
+
+def add_norm(resid: torch.Tensor, branch: Optional[torch.Tensor], w_post: Optional[torch.Tensor],
+             w_pre: Optional[torch.Tensor], out: Optional[torch.Tensor], *, eps_post: float = 0.0,
+             eps_pre: float = 0.0, off_post: float = 0.0, off_pre: float = 0.0,
+             rows: Optional[torch.Tensor] = None, n_partials: int = 1, full_precision: bool) -> None:
+    """resid += norm_post(sum of branch partials); out = norm_pre(resid).  Each piece is optional."""
+    if resid.dim() != 2:
+        raise HipLibraryError("resid must be [T, H]")
+    Tres, H = resid.shape
+    _dev(resid, "resid", torch.float32)
+    T = Tres if rows is None else rows.numel()
+    stride = 0
+    if branch is not None:
+        want = (n_partials, Tres, H) if n_partials > 1 else (Tres, H)
+        _dev(branch, "branch", torch.float32, want)
+        stride = Tres * H
+    elif n_partials != 1:
+        raise HipLibraryError("partial sums need a branch")
+    w_dtype = None
+    for w, nm in ((w_post, "w_post"), (w_pre, "w_pre")):
+        if w is not None:
+            _dev(w, nm, None, (H,))
+            if w_dtype is not None and w.dtype != w_dtype:
+                raise HipLibraryError("w_post and w_pre must have one dtype")
+            w_dtype = w.dtype
+    if w_post is not None and branch is None:
+        raise HipLibraryError("w_post without a branch")
+    if out is not None:
+        _dev(out, "out", None, (T, H))
+    elif w_pre is not None:
+        raise HipLibraryError("w_pre without an output")
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+    _call("alice_add_norm", resid.data_ptr(), _opt(branch, "branch"), n_partials, stride,
+          _opt(w_post, "w_post"), _opt(w_pre, "w_pre"), dtype_code(w_dtype or torch.float32),
+          _opt(out, "out"), dtype_code(out.dtype if out is not None else torch.float32),
+          _opt(rows, "rows"), T, H, float(eps_post), float(eps_pre), float(off_post), float(off_pre),
+          int(full_precision), _stream())
+
+
+def softcap_(x: torch.Tensor, cap: float, full_precision: bool) -> None:
+    _dev(x, "x", torch.float32)
+    _call("alice_softcap", x.data_ptr(), x.numel(), float(cap), int(full_precision), _stream())
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, n_out: int, k_in: int,
+           layout: int = LAYOUT_ROW, epilogue: int = EPI_NONE, epi_param: float = 0.0,
+           split_k: int = 1, variant: int = LINEAR_AUTO, full_precision: bool) -> None:
+    """y = x . W^T.  W: [n_out (2 n_out for GeGLU), k_in] row-major, or its fragment layout."""
+    if x.dim() != 2 or x.shape[1] != k_in:
+        raise HipLibraryError(f"x must be [M, {k_in}], found {tuple(x.shape)}")
+    M = x.shape[0]
+    _dev(x, "x")
+    w_rows = n_out * (2 if epilogue == EPI_GEGLU else 1)
+    if layout == LAYOUT_ROW:
+        _dev(w, "w", None, (w_rows, k_in))
+    else:
+        _dev(w, "w", torch.bfloat16)
+        need = ((w_rows + 15) // 16 * 16) * ((k_in + 31) // 32 * 32)
+        if w.numel() != need:
+            raise HipLibraryError(f"w in fragment layout must hold {need} elements, found {w.numel()}")
+    want = (split_k, M, n_out) if split_k > 1 else (M, n_out)
+    _dev(y, "y", None, want)
+    if split_k > 1 and y.dtype != torch.float32:
+        raise HipLibraryError("partial sums are float32")
+    _call("alice_linear", x.data_ptr(), dtype_code(x.dtype), w.data_ptr(), dtype_code(w.dtype), layout,
+          y.data_ptr(), dtype_code(y.dtype), M, n_out, k_in, epilogue, float(epi_param), split_k, variant,
+          int(full_precision), _stream())
+
+
+def linear_split_hint(M: int, N: int, K: int, layout: int) -> int:
+    return library().alice_linear_split_hint(M, N, K, layout)
+
+
+def to_frag16(w: torch.Tensor) -> torch.Tensor:
+    """A row-major bfloat16 [N, K] matrix rearranged into the fragment layout (flat, zero padded)."""
+    _dev(w, "w", torch.bfloat16)
+    if w.dim() != 2:
+        raise HipLibraryError("w must be [N, K]")
+    N, K = w.shape
+    out = torch.empty(((N + 15) // 16 * 16) * ((K + 31) // 32 * 32), dtype=torch.bfloat16, device=w.device)
+    _call("alice_to_frag16", w.data_ptr(), out.data_ptr(), N, K, _stream())
+    return out
+
+
+def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[torch.Tensor],
+                     v_pool: Optional[torch.Tensor], cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                     positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
+                     block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
+                     rotary_dim: int, max_position: int) -> None:
+    """Rotate q and k; write k and v at their positions into the pools [pages, nKV, page, d].
+    With k_pool None the row holds q only (num_kv_heads = 0) and nothing is cached.
+    `max_position` is the largest position among `positions` (the host knows it): checked against the tables."""
+    T = qkv.shape[0]
+    dt = qkv.dtype
+    _dev(qkv, "qkv")
+    row_width = qkv.shape[1]
+    if qkv.dim() != 2 or row_width < (num_heads + (2 * num_kv_heads if k_pool is not None else 0)) * head_dim:
+        raise HipLibraryError(f"qkv rows of {tuple(qkv.shape)} are too short for the heads")
+    _dev(q_out, "q_out", dt, (T, num_heads * head_dim))
+    _dev(positions, "positions", torch.int32, (T,))
+    if cos is not None:
+        if cos.dim() != 2 or cos.shape[1] != rotary_dim // 2 or sin.shape != cos.shape:
+            raise HipLibraryError(f"cos/sin tables must be [positions, {rotary_dim // 2}]")
+        _dev(cos, "cos", torch.float32)
+        _dev(sin, "sin", torch.float32)
+        if max_position >= cos.shape[0]:
+            raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({cos.shape[0]} positions)")
+    page_size = n_pages = bt_stride = 0
+    if k_pool is not None:
+        if k_pool.dim() != 4 or k_pool.shape[1] != num_kv_heads or k_pool.shape[3] != head_dim:
+            raise HipLibraryError(f"k_pool must be [pages, {num_kv_heads}, page, {head_dim}], found {tuple(k_pool.shape)}")
+        _dev(k_pool, "k_pool", dt)
+        _dev(v_pool, "v_pool", dt, k_pool.shape)
+        n_pages, _, page_size, _ = k_pool.shape
+        _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+        _dev(block_table, "block_table", torch.int32)
+        if block_table.dim() != 2:
+            raise HipLibraryError("block_table must be [sequences, pages per sequence]")
+        bt_stride = block_table.shape[1]
+        if max_position // page_size >= bt_stride:
+            raise HipLibraryError(f"position {max_position} is beyond the block table ({bt_stride} pages of {page_size})")
+    _call("alice_rope_cache_write", qkv.data_ptr(), dtype_code(dt), q_out.data_ptr(), _opt(k_pool, "k_pool"),
+          _opt(v_pool, "v_pool"), _opt(cos, "cos"), _opt(sin, "sin"), positions.data_ptr(),
+          _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T, row_width, num_heads,
+          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, _stream())
+
+
+def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor,
+                      positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, *,
+                      num_heads: int, scale: float, softcap: Optional[float], window: Optional[int],
+                      max_position: int, full_precision: bool) -> None:
+    T = q.shape[0]
+    dt = q.dtype
+    if k_pool.dim() != 4:
+        raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
+    n_pages, nKV, page_size, d = k_pool.shape
+    _dev(q, "q", None, (T, num_heads * d))
+    _dev(out, "out", dt, (T, num_heads * d))
+    _dev(k_pool, "k_pool", dt)
+    _dev(v_pool, "v_pool", dt, k_pool.shape)
+    _dev(positions, "positions", torch.int32, (T,))
+    _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"position {max_position} is beyond the block table {tuple(block_table.shape)}")
+    _call("alice_attention_generic", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), v_pool.data_ptr(),
+          out.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+          block_table.shape[1], T, num_heads, nKV, d, page_size, float(scale),
+          float(softcap or 0.0), int(window or 0), int(full_precision), _stream())
+
+
+def fragment_layout_available() -> bool:
+    """Whether this build of the library has the MFMA kernels that read the fragment layout."""
+    return bool(getattr(library(), "alice_has_mfma_linear", lambda: 0)())
+
+
+def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,
+              block_table: torch.Tensor, *, num_heads: int, scale: float, softcap: Optional[float],
+              window: Optional[int], full_precision: bool) -> None:
+    """Attention of the step's query tokens over the cache; picks the kernel for the step's shape.
+    `ctx` carries positions, seq_of_token, max_position (and the prompt/decode shape of the step)."""
+    attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
+                      num_heads=num_heads, scale=scale, softcap=softcap, window=window,
+                      max_position=ctx.max_position, full_precision=full_precision)

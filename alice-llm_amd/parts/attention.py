@@ -1,0 +1,77 @@
+"""The attention mixer: grouped-query attention over the paged cache.
+
+q, k, v projections (no biases), position encoding of q and k, k and v cached, then per query
+head h with kv head h // (nH // nKV): score = (q . k) * scale, softcap cap * tanh(s / cap),
+softmax over the keys max(0, pos + 1 - window) .. pos, weighted sum of v, output projection
+(llama3.rs:14206-14217, 14307-14331, 5431-5451, 5622-5688, 14423).  Scale, softcap, window, head
+counts and head size are constructor arguments; window None is global attention, softcap None
+turns the tanh off.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..hip import ops
+from .base import MIXERS, CacheNeed, KVNeed, ParamSpec, Part, Precision
+from .linear import Linear
+
+
+@MIXERS.register("attention")
+class Attention(Part):
+    def __init__(self, precision: Precision, positions: dict, *, hidden_size: int, num_heads: int,
+                 num_kv_heads: int, head_dim: int, scale: float, softcap: Optional[float] = None,
+                 window: Optional[int] = None, position: Optional[str] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
+        self.precision = precision
+        self.H, self.nH, self.nKV, self.d = hidden_size, num_heads, num_kv_heads, head_dim
+        self.scale = float(scale)
+        self.softcap = None if softcap is None else float(softcap)
+        self.window = window
+        self.position = positions[position] if position is not None else positions.get("none")
+        if self.position is None:
+            raise ValueError("attention needs a position encoding (use 'none' for no rotation)")
+        self.q_dim, self.kv_dim = num_heads * head_dim, num_kv_heads * head_dim
+        self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, precision)
+        self.o = Linear(self.q_dim, hidden_size, precision)
+        self._parts: Dict[str, torch.Tensor] = {}
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"q_proj.weight": ParamSpec((self.q_dim, self.H)),
+                "k_proj.weight": ParamSpec((self.kv_dim, self.H)),
+                "v_proj.weight": ParamSpec((self.kv_dim, self.H)),
+                "o_proj.weight": ParamSpec((self.H, self.q_dim))}
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window))
+
+    def assign(self, name: str, tensor: torch.Tensor) -> None:
+        if name == "o_proj.weight":
+            self.o.load(tensor)
+        elif name in ("q_proj.weight", "k_proj.weight", "v_proj.weight"):
+            self._parts[name] = tensor
+        else:
+            raise KeyError(name)
+
+    def finalize(self) -> None:
+        q, k, v = (self._parts.pop(n + "_proj.weight") for n in "qkv")
+        if not (q.dtype == k.dtype == v.dtype):
+            q, k, v = q.float(), k.float(), v.float()       # one stored in 32-bit: the fused matrix stays 32-bit
+        self.qkv.load(torch.cat([q, k, v], dim=0))          # rows: all q heads, then k heads, then v heads
+
+    def weight_bytes(self) -> int:
+        return self.qkv.nbytes() + self.o.nbytes()
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """x: [T, H] in the activation dtype; returns the branch in float32 ([T, H] or partial sums)."""
+        T = x.shape[0]
+        qkv = self.qkv(x, self.precision.act)
+        q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
+        self.position.rotate_and_store(qkv, q, ctx, cache, num_heads=self.nH, num_kv_heads=self.nKV,
+                                       head_dim=self.d)
+        out = torch.empty_like(q)
+        ops.attention(q, cache.k, cache.v, out, ctx, cache.block_table, num_heads=self.nH, scale=self.scale,
+                      softcap=self.softcap, window=self.window, full_precision=self.precision.full)
+        return self.o(out, torch.float32, allow_partials=True)

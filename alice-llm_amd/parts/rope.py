@@ -1,0 +1,59 @@
+"""Position encodings.  Rotary, half-split pairing (j, j + R/2) over the rotated width R:
+angle = position * theta^(-2j/R) (llama3.rs:5367-5378; same pairing in src/rope.rs:12-27).
+
+The angles' cosines and sines are tabulated once on the host in 64-bit and stored as 32-bit, so
+the rotation itself is a 32-bit multiply-add in the kernel.  A position encoding serves the
+attention mixer through `rotate_and_store`: rotate q and k, and put k and v into the cache in the
+same pass, which saves one trip through memory for k.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..hip import ops
+from .base import POSITIONS, Part, Precision
+
+
+@POSITIONS.register("rope")
+class RotaryEncoding(Part):
+    def __init__(self, precision: Precision, device, *, dim: int, theta: float, max_positions: int,
+                 rotary_dim: Optional[int] = None):
+        self.dim = dim
+        self.rotary_dim = dim if rotary_dim is None else rotary_dim
+        if self.rotary_dim % 2 or self.rotary_dim > dim:
+            raise ValueError(f"rotated width {self.rotary_dim} must be even and at most {dim}")
+        self.theta = float(theta)
+        self.max_positions = max_positions
+        half = self.rotary_dim // 2
+        j = torch.arange(half, dtype=torch.float64)
+        inv_freq = self.theta ** (-2.0 * j / self.rotary_dim)
+        ang = torch.arange(max_positions, dtype=torch.float64)[:, None] * inv_freq[None, :]
+        self.cos = torch.cos(ang).to(torch.float32).to(device).contiguous()
+        self.sin = torch.sin(ang).to(torch.float32).to(device).contiguous()
+
+    def rotate_and_store(self, qkv: torch.Tensor, q_out: torch.Tensor, ctx, cache, *, num_heads: int,
+                         num_kv_heads: int, head_dim: int) -> None:
+        write = cache is not None and cache.writable
+        ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None,
+                             self.cos, self.sin, ctx.positions, ctx.seq_of_token if write else None,
+                             cache.block_table if write else None, num_heads=num_heads,
+                             num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=self.rotary_dim,
+                             max_position=ctx.max_position)
+
+
+@POSITIONS.register("none")
+class NoPositionEncoding(Part):
+    """No rotation: q passes through, k and v go to the cache unchanged."""
+
+    def __init__(self, precision: Precision, device, **_):
+        pass
+
+    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim) -> None:
+        write = cache is not None and cache.writable
+        ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None, None, None,
+                             ctx.positions, ctx.seq_of_token if write else None,
+                             cache.block_table if write else None, num_heads=num_heads,
+                             num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=0,
+                             max_position=ctx.max_position)
