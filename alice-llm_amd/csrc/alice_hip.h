@@ -60,6 +60,13 @@ int alice_attention_generic(const void* q, int dtype, const void* k_pool, const 
                             int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
                             float softcap, int window, int full_precision, hipStream_t stream);
 
+// Lowest index among equal maxima.
+int alice_argmax(const float* logits, int* out, int B, int V, hipStream_t stream);
+// temperature -> top-k (0: off) -> top-p (>= 1: off) -> softmax -> first index whose cumulative
+// probability exceeds uniform[row].
+int alice_sample(const float* logits, int* out, const float* uniform, int B, int V, float temperature,
+                 int top_k, float top_p, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 

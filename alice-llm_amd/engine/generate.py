@@ -1,7 +1,126 @@
-"""placeholder"""
-from dataclasses import dataclass
+"""The generation loop above the step function: batches of unequal prompts, stop tokens, sequences
+that end earlier, and as many batches one after another as there are requests.
+
+A batch starts together: one step runs all its prompts, then every live sequence gets one token per
+step.  A sequence ends when it draws a stop token (which is not part of its output, as in the
+reference, llama3.rs:16137-16139) or reaches its own cap of new tokens (llama3.rs:17813-17835); it
+leaves the batch at once and its slot goes back to the cache, where the next batch takes it.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, List, Optional, Sequence
+
+PAGE = 64
+
+
 @dataclass
 class GenerationResult:
-    tokens: list
+    tokens: List[int]
+    finish_reason: str              # "stop": a stop token was drawn; "length": the cap was reached
+    prompt_tokens: int
+    prefill_ms: float = 0.0         # of the batch the request ran in
+    decode_ms: float = 0.0
+
+    @property
+    def tokens_generated(self) -> int:
+        return len(self.tokens)
+
+
+def plan_batches(prompt_lens: Sequence[int], caps: Sequence[int], *, max_batch: Optional[int],
+                 capacity_tokens: int, max_slots: int, page: int = PAGE) -> List[List[int]]:
+    """Split requests, in order, into batches that fit: at most max_batch (and max_slots) sequences,
+    and room in the cache for every sequence at its longest, each rounded up to whole pages."""
+    limit = min(max_batch or max_slots, max_slots)
+    batches: List[List[int]] = []
+    cur: List[int] = []
+    used = 0
+    for i, (n, c) in enumerate(zip(prompt_lens, caps)):
+        need = -(-(n + max(c, 0)) // page) * page
+        if need > capacity_tokens:
+            raise ValueError(f"request {i} needs room for {need} tokens, the cache holds {capacity_tokens}")
+        if cur and (len(cur) >= limit or used + need > capacity_tokens):
+            batches.append(cur)
+            cur, used = [], 0
+        cur.append(i)
+        used += need
+    if cur:
+        batches.append(cur)
+    return batches
+
+
 class Generator:
-    pass
+    """Runs requests through an engine.  `engine` needs open(n), step(slots, tokens, want) and
+    close(slots) and a cache with `max_tokens` and `slots.n_slots`; `sampler(logits, requests, draws)`
+    returns one token id per row (anything with .tolist())."""
+
+    def __init__(self, engine, *, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
+                 stop_token_ids: Sequence[int] = (), max_batch: Optional[int] = None,
+                 sampler: Optional[Callable] = None, include_stop_token: bool = False):
+        self.engine = engine
+        if sampler is None:
+            from ..sampling import Sampler
+            sampler = Sampler(temperature, top_k, top_p, seed)
+        self.sampler = sampler
+        self.stop = set(int(t) for t in stop_token_ids)
+        self.max_batch = max_batch
+        self.include_stop_token = include_stop_token
+
+    def run(self, prompts: Sequence[Sequence[int]], max_new_tokens: Sequence[int]) -> List[GenerationResult]:
+        if len(prompts) != len(max_new_tokens):
+            raise ValueError("one cap of new tokens per prompt")
+        if any(len(p) == 0 for p in prompts):
+            raise ValueError("every prompt needs at least one token")
+        results: List[Optional[GenerationResult]] = [None] * len(prompts)
+        cache = self.engine.cache
+        batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch=self.max_batch,
+                               capacity_tokens=cache.max_tokens, max_slots=cache.slots.n_slots)
+        for batch in batches:
+            self._run_batch(batch, prompts, max_new_tokens, results)
+        return results  # type: ignore[return-value]
+
+    def _run_batch(self, batch, prompts, caps, results) -> None:
+        eng = self.engine
+        out = {r: [] for r in batch}
+        reason = {}
+        live = [r for r in batch if caps[r] > 0]
+        for r in batch:
+            if caps[r] <= 0:
+                reason[r] = "length"
+        slots = dict(zip(live, eng.open(len(live))))
+        t0 = time.perf_counter()
+        prefill_ms = 0.0
+        try:
+            feed = [list(prompts[r]) for r in live]
+            first = True
+            while live:
+                logits = eng.step([slots[r] for r in live], feed, "last")
+                ids = self.sampler(logits, live, [len(out[r]) for r in live]).tolist()   # waits for the step
+                if first:
+                    prefill_ms = (time.perf_counter() - t0) * 1e3
+                    first = False
+                still, feed = [], []
+                for r, tok in zip(live, ids):
+                    tok = int(tok)
+                    if tok in self.stop:
+                        if self.include_stop_token:
+                            out[r].append(tok)
+                        reason[r] = "stop"
+                    else:
+                        out[r].append(tok)
+                        if len(out[r]) >= caps[r]:
+                            reason[r] = "length"
+                    if r in reason:
+                        eng.close([slots.pop(r)])            # the slot is free for the next batch at once
+                    else:
+                        still.append(r)
+                        feed.append([tok])
+                live = still
+        finally:
+            if slots:
+                eng.close(list(slots.values()))
+        decode_ms = (time.perf_counter() - t0) * 1e3 - prefill_ms
+        for r in batch:
+            results[r] = GenerationResult(tokens=out[r], finish_reason=reason[r], prompt_tokens=len(prompts[r]),
+                                          prefill_ms=prefill_ms, decode_ms=decode_ms)

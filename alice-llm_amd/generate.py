@@ -1,0 +1,108 @@
+"""Command line: python -m alice_llm_amd.generate --model DIR --prompt-ids 2,651,9456 --max-tokens 32
+
+Option names and meanings follow the reference's generate examples where it has them
+(--model, --max-tokens default 256, --temperature, --top-k: examples/elyza_gguf.rs:81-117 and
+examples/generate_gpu.rs:31-40; temperature 0 is greedy, generate_gpu.rs:122; --logits-dump N writes
+the top-5 logits of the first N generated positions as JSON lines to stderr,
+examples/elyza_gguf.rs:31-76).  There is no tokenizer here: prompts are token ids, and so is the
+output.  The closing lines are the reference's (examples/elyza_gguf.rs:277-286).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+from typing import List
+
+
+def _ids(text: str) -> List[int]:
+    return [int(t) for t in text.replace(",", " ").split()]
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="python -m alice_llm_amd.generate", description=__doc__,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", help="folder with config.json and model.safetensors")
+    ap.add_argument("--random-weights", action="store_true", help="random weights from --preset/--config and --weights-seed")
+    ap.add_argument("--preset", help="a named configuration (with --random-weights)")
+    ap.add_argument("--config", help="a config.json file (with --random-weights)")
+    ap.add_argument("--weights-seed", type=int, default=0)
+    ap.add_argument("--prompt-ids", action="append", default=[], help="token ids '1,2,3'; repeat for a batch")
+    ap.add_argument("--prompt-file", action="append", default=[], help="file with one prompt's token ids per line")
+    ap.add_argument("--max-tokens", type=int, default=256, help="cap on new tokens per sequence")
+    ap.add_argument("--temperature", type=float, default=0.0, help="0 is greedy")
+    ap.add_argument("--top-k", type=int, default=0, help="keep the k most likely tokens (0: off)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="nucleus mass (1: off)")
+    ap.add_argument("--seed", type=int, default=0, help="sampler seed")
+    ap.add_argument("--stop-ids", default=None, help="stop token ids '1,107' (default: the configuration's eos)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32", "bf16", "fp32"], default=None)
+    ap.add_argument("--max-batch", type=int, default=None, help="most sequences in one batch")
+    ap.add_argument("--logits-dump", type=int, default=0, help="dump top-5 logits of the first N generated positions")
+    args = ap.parse_args(argv)
+
+    import alice_llm_amd as alice
+
+    prompts = [_ids(p) for p in args.prompt_ids]
+    for path in args.prompt_file:
+        with open(path) as f:
+            prompts += [_ids(line) for line in f if line.strip()]
+    if not prompts:
+        ap.error("give at least one prompt with --prompt-ids or --prompt-file")
+    if args.random_weights:
+        if args.config:
+            with open(args.config) as f:
+                raw = json.load(f)
+        elif args.preset:
+            raw = alice.preset(args.preset)
+        else:
+            ap.error("--random-weights needs --preset or --config")
+        print(f"Building random weights (seed {args.weights_seed})", flush=True)
+        model = alice.load(raw, dtype=args.dtype, random_seed=args.weights_seed)
+    else:
+        if not args.model:
+            ap.error("give --model DIR, or --random-weights with --preset/--config")
+        print(f"Loading model: {args.model}", flush=True)
+        model = alice.load(args.model, dtype=args.dtype)
+
+    stop = _ids(args.stop_ids) if args.stop_ids is not None else None
+    if args.logits_dump > 0:
+        _dump_logits(model, prompts, args.logits_dump)
+    results = model.generate(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
+                             top_k=args.top_k, top_p=args.top_p, seed=args.seed, stop_token_ids=stop,
+                             max_batch=args.max_batch)
+    for i, r in enumerate(results):
+        print(f"[{i}] " + ",".join(str(t) for t in r.tokens) + f"  ({r.finish_reason})")
+    print("---")
+    g = sum(r.tokens_generated for r in results)
+    p = sum(r.prompt_tokens for r in results)
+    seen, prefill, decode = set(), 0.0, 0.0
+    for r in results:                       # times are per batch; count each batch once
+        key = (r.prefill_ms, r.decode_ms)
+        if key not in seen:
+            seen.add(key)
+            prefill += r.prefill_ms
+            decode += r.decode_ms
+    print(f"Tokens: {g} generated, {p} prompt")
+    tps = g / (decode / 1e3) if decode > 0 else 0.0
+    print(f"Speed: {tps:.1f} tok/s ({prefill:.0f} prefill + {decode:.0f} decode = {prefill + decode:.0f} total ms)")
+    return 0
+
+
+def _dump_logits(model, prompts, n: int) -> None:
+    """Greedy replay of the first prompt, one JSON line per position: the prompt's end, then n - 1 decoded tokens."""
+    import torch
+    eng = model.engine(max_tokens=-(-(len(prompts[0]) + n) // 64) * 64, max_seqs=1)
+    slot = eng.open(1)
+    feed = list(prompts[0])
+    for i in range(n):
+        logits = eng.step(slot, [feed], "last")[0]
+        top = torch.topk(logits, min(5, logits.numel()))
+        print(json.dumps({"position": eng.length(slot[0]) - 1,
+                          "top5": [[int(j), float(v)] for v, j in zip(top.values.tolist(), top.indices.tolist())]}),
+              file=sys.stderr, flush=True)
+        feed = [int(top.indices[0])]
+    eng.close(slot)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -43,6 +43,8 @@ def _declare(lib) -> None:
         "alice_to_frag16": [P, P, I, I, P],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
+        "alice_argmax": [P, P, I, I, P],
+        "alice_sample": [P, P, P, I, I, F, I, F, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -304,3 +306,28 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
                       max_position=ctx.max_position, full_precision=full_precision)
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """int32 [B]: index of each row's maximum, the lowest index among equal maxima."""
+    _dev(logits, "logits", torch.float32)
+    B, V = logits.shape
+    if out is None:
+        out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    _dev(out, "out", torch.int32, (B,))
+    _call("alice_argmax", logits.data_ptr(), out.data_ptr(), B, V, _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, uniform: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """int32 [B]: temperature, top-k, top-p, softmax and inverse CDF with uniform[row] in [0, 1)."""
+    _dev(logits, "logits", torch.float32)
+    B, V = logits.shape
+    _dev(uniform, "uniform", torch.float32, (B,))
+    if out is None:
+        out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    _dev(out, "out", torch.int32, (B,))
+    _call("alice_sample", logits.data_ptr(), out.data_ptr(), uniform.data_ptr(), B, V, float(temperature),
+          int(top_k), float(top_p), _stream())
+    return out

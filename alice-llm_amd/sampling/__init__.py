@@ -1,0 +1,1 @@
+from .sampler import Sampler, splitmix64, uniform, GREEDY_BELOW

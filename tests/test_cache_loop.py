@@ -1,0 +1,184 @@
+"""The cache's bookkeeping and the generation loop's decisions (no GPU)."""
+import random
+
+import pytest
+import torch
+
+from alice_llm_amd.cache import Cache, CacheError, SlotTable
+from alice_llm_amd.engine.generate import Generator, plan_batches
+from alice_llm_amd.parts import CacheNeed, KVNeed, StateNeed
+from alice_llm_amd.sampling import uniform
+
+
+def needs(window=8):
+    return [CacheNeed(kv=KVNeed(1, 16, window)), CacheNeed(kv=KVNeed(1, 16, None)), CacheNeed(kv=KVNeed(1, 16, window)), None]
+
+
+def make(max_tokens=640, window=8, **kw):
+    return Cache(needs(window), max_tokens=max_tokens, dtype=torch.float32, device="cpu", allocate=False, **kw)
+
+
+def test_slot_table():
+    t = SlotTable(3)
+    a, b, c = t.take(), t.take(), t.take()
+    assert sorted([a, b, c]) == [0, 1, 2] and t.n_free() == 0
+    with pytest.raises(CacheError, match="all 3 slots"):
+        t.take()
+    t.give_back(b)
+    with pytest.raises(CacheError, match="freed twice"):
+        t.give_back(b)
+    assert t.take() == b and t.length(b) == 0
+    t.advance(a, 5)
+    assert t.length(a) == 5 and t.held() == [0, 1, 2]
+    with pytest.raises(CacheError):
+        t.length(7)
+
+
+def test_groups_by_need():
+    c = make()
+    assert [g.layers for g in c.groups] == [[0, 2], [1]] and [g.need.window for g in c.groups] == [8, None]
+    assert c.max_tokens == 640 and c.groups[0].n_pages == 10
+
+
+def test_pages_grow_trim_and_return():
+    c = make(max_tokens=640, window=70)
+    s = c.open()
+    c.reserve([s], [200]); c.commit([s], [200])
+    win, glob = c.groups
+    assert len([p for p in glob.table(s) if p >= 0]) == 4
+    # next query at 200 reads keys 131..200: pages 0 and 1 (positions 0..127) are out of reach
+    assert [p >= 0 for p in win.table(s)] == [False, False, True, True]
+    assert win.n_free() == 8 and glob.n_free() == 6
+    c.check_consistent()
+    c.reserve([s], [1]); c.commit([s], [1])
+    assert c.length(s) == 201 and len(win.table(s)) == 4
+    rows = c.block_table_rows(0, [s], 6)
+    assert rows[0][:2] == [0, 0] and rows[0][4:] == [0, 0] and all(p > 0 for p in rows[0][2:4])
+    c.close(s)
+    assert win.n_free() == 10 and glob.n_free() == 10
+    with pytest.raises(CacheError):
+        c.close(s)
+    c.check_consistent()
+
+
+def test_capacity_error_before_any_change():
+    c = make(max_tokens=256)
+    a, b = c.open(), c.open()
+    c.reserve([a, b], [100, 60]); c.commit([a, b], [100, 60])          # 2 + 1 pages of 4
+    before = ([list(g.table(a)) for g in c.groups], [g.n_free() for g in c.groups])
+    with pytest.raises(CacheError, match="cache is full"):
+        c.reserve([a, b], [1, 100])                                      # b would need 2 more, 1 is free
+    assert ([list(g.table(a)) for g in c.groups], [g.n_free() for g in c.groups]) == before
+    with pytest.raises(CacheError, match="twice"):
+        c.reserve([a, a], [1, 1])
+    c.check_consistent()
+
+
+def test_random_traffic_loses_nothing():
+    rng = random.Random(0)
+    c = make(max_tokens=64 * 40, window=100, max_seqs=6)
+    live = {}
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and c.slots.n_free():
+            live[c.open()] = 0
+        elif op < 0.45 and live:
+            s = rng.choice(list(live)); c.close(s); del live[s]
+        elif live:
+            ss = rng.sample(list(live), rng.randint(1, len(live)))
+            ns = [rng.choice([1, 1, 1, 7, 64, 130]) for _ in ss]
+            try:
+                c.reserve(ss, ns)
+            except CacheError:
+                continue
+            c.commit(ss, ns)
+            for s, n in zip(ss, ns):
+                live[s] += n
+        c.check_consistent()
+        assert all(c.length(s) == n for s, n in live.items())
+    for s in list(live):
+        c.close(s)
+    c.check_consistent()
+    assert all(g.n_free() == g.n_pages for g in c.groups) and c.slots.n_free() == 6
+
+
+def test_state_region_is_zeroed_on_open():
+    c = Cache([CacheNeed(state=StateNeed((3, 2)))], max_tokens=128, dtype=torch.float32, device="cpu", max_seqs=2)
+    assert c.state[0].shape == (2, 3, 2) and not c.groups
+    s = c.open(); c.state[0][s] += 5; c.close(s)
+    s2 = c.open()
+    assert s2 == s and float(c.state[0][s2].abs().sum()) == 0.0
+
+
+# ------------------------------------------------------------------ the loop
+class FakeEngine:
+    """Scripted logits: token = (last token fed + 1) mod V for every sequence; records slot traffic."""
+
+    def __init__(self, V=16, max_tokens=64 * 8, n_slots=4):
+        self.V = V
+        self.cache = make(max_tokens=max_tokens, max_seqs=n_slots)
+        self.opened, self.closed, self.steps = [], [], []
+
+    def open(self, n):
+        s = [self.cache.open() for _ in range(n)]
+        self.opened += s
+        return s
+
+    def close(self, slots):
+        for s in slots:
+            self.cache.close(s)
+        self.closed += list(slots)
+
+    def step(self, slots, tokens, want):
+        self.cache.reserve(slots, [len(t) for t in tokens]); self.cache.commit(slots, [len(t) for t in tokens])
+        self.steps.append((list(slots), [len(t) for t in tokens]))
+        out = torch.zeros(len(slots), self.V)
+        for i, t in enumerate(tokens):
+            out[i, (t[-1] + 1) % self.V] = 1.0
+        return out
+
+
+def argmax_sampler(logits, requests, draws):
+    return logits.argmax(-1)
+
+
+def test_plan_batches():
+    assert plan_batches([5, 12, 17, 100], [8] * 4, max_batch=2, capacity_tokens=256, max_slots=4) == [[0, 1], [2, 3]]
+    assert plan_batches([60, 60, 60], [10] * 3, max_batch=None, capacity_tokens=256, max_slots=8) == [[0, 1], [2]]
+    with pytest.raises(ValueError, match="request 1"):
+        plan_batches([5, 300], [8, 8], max_batch=4, capacity_tokens=256, max_slots=4)
+
+
+def test_loop_stop_tokens_caps_and_slot_reuse():
+    eng = FakeEngine()
+    gen = Generator(eng, stop_token_ids=[9], max_batch=2, sampler=argmax_sampler)
+    prompts = [[1, 2, 3], [7], [4, 5], [12, 13, 14, 15], [2]]
+    caps = [4, 10, 0, 3, 2]
+    res = gen.run(prompts, caps)
+    assert [r.tokens for r in res] == [[4, 5, 6, 7], [8], [], [0, 1, 2], [3, 4]]
+    assert [r.finish_reason for r in res] == ["length", "stop", "length", "length", "length"]     # 9 is not appended
+    assert [r.prompt_tokens for r in res] == [3, 1, 2, 4, 1]
+    # first step of a batch brings whole prompts of unequal length, later steps one token each; the batch shrinks
+    assert eng.steps[0] == ([0, 1], [3, 1]) and eng.steps[1][1] == [1, 1] and eng.steps[2] == ([0], [1])
+    assert sorted(eng.opened) == sorted(eng.closed) and len(eng.opened) == 4       # cap 0 takes no slot
+    assert set(eng.opened) <= {0, 1}                                                # later batches use the same slots again
+    eng.cache.check_consistent()
+    assert eng.cache.slots.n_free() == 4
+    gen2 = Generator(FakeEngine(), stop_token_ids=[9], sampler=argmax_sampler, include_stop_token=True)
+    assert gen2.run([[7]], [10])[0].tokens == [8, 9]
+
+
+def test_loop_gives_slots_back_on_error():
+    eng = FakeEngine(max_tokens=128)
+    def bad_sampler(logits, requests, draws):
+        raise RuntimeError("boom")
+    with pytest.raises(RuntimeError):
+        Generator(eng, sampler=bad_sampler).run([[1], [2]], [3, 3])
+    assert eng.cache.slots.n_free() == 4
+    eng.cache.check_consistent()
+
+
+def test_uniform_stream_is_per_request():
+    a = [uniform(7, 3, n) for n in range(5)]
+    assert a == [uniform(7, 3, n) for n in range(5)] and all(0 <= u < 1 for u in a)
+    assert a != [uniform(8, 3, n) for n in range(5)] and a != [uniform(7, 4, n) for n in range(5)]
