@@ -1,7 +1,7 @@
 """The cache: a slot per sequence, keys and values per layer in pages, and fixed-size state.
 
-Layers are grouped by what they need: all layers that keep every key form one group, all layers
-that read a window of W keys form another, each with page storage of its own
+The runs of the schedule (one per layer, unless the schedule names a layer twice) are grouped by what
+they need: all that keep every key form one group, all that read a window of W keys form another, each with page storage of its own
 ([layers of the group][page][kv head][64 positions][head_dim]) and a page table per slot.  A
 windowed group gives pages back as soon as no later query can reach them.  A slot is taken when a
 sequence starts and given back when it ends; its pages return to the pools and are used again
@@ -141,7 +141,7 @@ class LayerCache:
 class Cache:
     def __init__(self, needs: Sequence[Optional[CacheNeed]], *, max_tokens: int, dtype: torch.dtype, device,
                  max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE, allocate: bool = True):
-        """needs[i]: what layer i declares (None: nothing).  `max_tokens`: the most tokens that live
+        """needs[i]: what run i of the schedule declares (None: nothing).  `max_tokens`: the most tokens that live
         sequences hold at any time, each sequence's count rounded up to a multiple of the page size."""
         self.page_size = page_size
         self.device = device

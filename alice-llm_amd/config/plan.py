@@ -43,8 +43,10 @@ class LayerPlan:
 
 @dataclass(frozen=True)
 class ScheduleEntry:
-    """One run of a layer.  `cache_from` names the layer whose cache this run reads
-    instead of writing its own (the reference's kv_layer_map, llama3.rs:4739-4745)."""
+    """One run of a layer.  Every run owns cache storage of its own (a layer named twice keeps two
+    caches, one per run), unless `cache_from` names an earlier entry of the schedule, by its index,
+    whose cache this run reads instead of writing one (the reference's kv_layer_map,
+    llama3.rs:4739-4745)."""
     layer: int
     cache_from: Optional[int] = None
 

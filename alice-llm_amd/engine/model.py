@@ -42,10 +42,19 @@ class CausalLM:
         self.layers: List[Layer] = [Layer(lp, p, self.positions) for lp in plan.layers]
         self.final_norm = NORMS.get(plan.final_norm.kind)(p, **plan.final_norm.args) if plan.final_norm else None
         self.head = HEADS.get(plan.head.kind)(p, **plan.head.args)
-        for e in plan.schedule:
-            if not 0 <= e.layer < len(self.layers) or (e.cache_from is not None
-                                                       and not 0 <= e.cache_from < len(self.layers)):
-                raise ValueError(f"schedule entry {e} names a layer that does not exist")
+        for i, e in enumerate(plan.schedule):
+            if not 0 <= e.layer < len(self.layers):
+                raise ValueError(f"schedule entry {i} names layer {e.layer}, which does not exist")
+            if e.cache_from is not None:
+                if not 0 <= e.cache_from < i or plan.schedule[e.cache_from].cache_from is not None:
+                    raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_from}, which must be "
+                                     f"an earlier entry with a cache of its own")
+                a, b = self._need(e.layer), self._need(plan.schedule[e.cache_from].layer)
+                if a is None or b is None or a.kv is None or b.kv is None or \
+                        (a.kv.num_kv_heads, a.kv.head_dim) != (b.kv.num_kv_heads, b.kv.head_dim) or \
+                        (b.kv.window is not None and (a.kv.window is None or a.kv.window > b.kv.window)):
+                    raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_from}: "
+                                     f"its keys differ in shape or reach further back than that cache keeps")
         self._loaded = False
 
     # ------------------------------------------------------------------ parameters
@@ -94,8 +103,13 @@ class CausalLM:
         return total
 
     # ------------------------------------------------------------------ cache needs
+    def _need(self, layer: int):
+        mixer = self.layers[layer].mixer
+        return mixer.cache_need() if hasattr(mixer, "cache_need") else None
+
     def cache_needs(self):
-        return [layer.mixer.cache_need() if hasattr(layer.mixer, "cache_need") else None for layer in self.layers]
+        """What each entry of the schedule needs from the cache (None for a run that reads another's)."""
+        return [None if e.cache_from is not None else self._need(e.layer) for e in self.plan.schedule]
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, cache, block_tables) -> torch.Tensor:
@@ -103,8 +117,8 @@ class CausalLM:
         if not self._loaded:
             raise RuntimeError("the model has no weights yet")
         stream = ResidualStream(self.embedding.forward(ctx.tokens), self.precision)
-        for entry in self.plan.schedule:
-            view = cache.view(entry.layer, block_tables, read_from=entry.cache_from)
+        for i, entry in enumerate(self.plan.schedule):
+            view = cache.view(i, block_tables, read_from=entry.cache_from)
             self.layers[entry.layer].block.forward(stream, ctx, view)
         if ctx.want_rows is None or ctx.want_rows.numel() == 0:
             stream.flush()

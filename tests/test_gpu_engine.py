@@ -1,0 +1,165 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16: whole requests, the last 32
+tokens one by one, unequal batches one after another on reused slots, long decoding, first tokens."""
+import pytest
+import torch
+
+import alice_llm_amd as alice
+from helpers import TINY, TOL, max_err, model_folder, plain_model, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+CASES = [(n, d) for n in ("tiny-a", "tiny-b", "tiny-c") for d in ("float32", "bfloat16")]
+_MODELS = {}
+
+
+def setup(name, dtype, stored="bfloat16", hot=1.0):
+    key = (name, dtype, stored, hot)
+    if key not in _MODELS:
+        folder = model_folder(name, stored, hot)
+        _MODELS[key] = (alice.load(folder, dtype=dtype), plain_model(folder))
+    return _MODELS[key]
+
+
+def tol(dtype, ref):
+    return TOL[dtype] * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_each_request_alone_and_whole(name, dtype):
+    model, plain = setup(name, dtype)
+    eng = model.engine(max_tokens=512)
+    for n, seed in ((1, 1), (2, 2), (9, 3), (64, 4), (65, 5), (200, 6)):
+        toks = random_tokens(plain.V, n, seed)
+        ref = plain.forward(toks)
+        s = eng.open(1)
+        got = eng.step(s, [toks], "all")
+        eng.close(s)
+        assert got.shape == ref.shape and got.dtype == torch.float32
+        assert max_err(got, ref) < tol(dtype, ref), (n, max_err(got, ref))
+    eng.cache.check_consistent()
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_last_32_tokens_one_by_one(name, dtype):
+    model, plain = setup(name, dtype)
+    eng = model.engine(max_tokens=256)
+    toks = random_tokens(plain.V, 150, 7)
+    ref = plain.forward(toks)
+    s = eng.open(1)
+    got = [eng.step(s, [toks[:-32]], "all")]
+    for t in toks[-32:]:
+        got.append(eng.step(s, [[t]], "last"))
+    eng.close(s)
+    got = torch.cat(got)
+    assert max_err(got, ref) < tol(dtype, ref)
+    # the two ways of cutting agree with each other more closely than with the 64-bit oracle
+    s = eng.open(1)
+    whole = eng.step(s, [toks], "all")
+    eng.close(s)
+    assert max_err(got, whole) < (1e-5 if dtype == "float32" else tol(dtype, ref))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_unequal_batches_on_reused_slots(name, dtype):
+    model, plain = setup(name, dtype)
+    eng = model.engine(max_tokens=64 * 8, max_seqs=4)
+    worst = 0.0
+    for batch_no, lens in enumerate(((5, 12, 17), (3, 70, 14, 21), (130, 2))):
+        seqs = [random_tokens(plain.V, n + 6 + 3 * i, 10 * batch_no + i) for i, n in enumerate(lens)]
+        refs = [plain.forward(s) for s in seqs]
+        slots = eng.open(len(seqs))
+        assert set(slots) <= {0, 1, 2, 3}
+        got = eng.step(slots, [s[:n] for s, n in zip(seqs, lens)], "all")      # prompts of unequal length, one step
+        ref = torch.cat([r[:n] for r, n in zip(refs, lens)])
+        worst = max(worst, max_err(got, ref) / tol(dtype, ref))
+        live = list(range(len(seqs)))
+        step = 0
+        while live:                                                              # then one token each; shorter ones end earlier
+            feed = [[seqs[i][lens[i] + step]] for i in live]
+            got = eng.step([slots[i] for i in live], feed, "last")
+            ref = torch.stack([refs[i][lens[i] + step] for i in live])
+            worst = max(worst, max_err(got, ref) / tol(dtype, ref))
+            step += 1
+            done = [i for i in live if lens[i] + step >= len(seqs[i])]
+            eng.close([slots[i] for i in done])
+            live = [i for i in live if i not in done]
+        eng.cache.check_consistent()
+    assert worst < 1.0, worst
+    assert eng.cache.slots.n_free() == 4
+
+
+@pytest.mark.parametrize("name,dtype", [("tiny-a", "float32"), ("tiny-b", "bfloat16"), ("tiny-c", "bfloat16"), ("tiny-c", "float32")])
+def test_long_decoding_across_pages_and_window(name, dtype):
+    model, plain = setup(name, dtype)
+    eng = model.engine(max_tokens=64 * 6, max_seqs=2)
+    toks = random_tokens(plain.V, 300, 11)
+    ref = plain.forward(toks)
+    s = eng.open(2)                               # a second sequence keeps the batch mixed
+    other = random_tokens(plain.V, 40, 12)
+    got = [eng.step(s, [toks[:3], other], [[0, 1, 2], []])]
+    got.append(eng.step([s[0]], [[toks[3]]], "last"))
+    eng.close([s[1]])
+    for t in toks[4:]:
+        got.append(eng.step([s[0]], [[t]], "last"))
+    got = torch.cat(got)
+    assert max_err(got, ref) < tol(dtype, ref)
+    win = [g for g in eng.cache.groups if g.need.window is not None][0]
+    assert sum(p >= 0 for p in win.table(s[0])) < 5 - (win.need.window < 64)    # the window gave pages back
+    eng.close([s[0]])
+    eng.cache.check_consistent()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_hot_weights_reach_the_caps(dtype):
+    # With N(0, 0.02) weights scores and logits stay far below the caps; this variant multiplies q, k and
+    # the embedding so that both tanh stages bend the values.
+    model, plain = setup("tiny-b", dtype, hot=12.0)
+    toks = random_tokens(plain.V, 40, 13)
+    ref = plain.forward(toks)
+    uncapped = plain_model_without_caps(plain).forward(toks)
+    assert (uncapped - ref).abs().max() > 0.5, "the caps do not bite in this variant"
+    eng = model.engine(max_tokens=128)
+    s = eng.open(1)
+    got = eng.step(s, [toks], "all")
+    eng.close(s)
+    assert max_err(got, ref) < tol(dtype, ref) * (1 if dtype == "float32" else 3), max_err(got, ref)
+
+
+def plain_model_without_caps(plain):
+    import copy
+    p = copy.copy(plain)
+    p.cap_a = None
+    p.cap_f = None
+    return p
+
+
+def test_stored_float32_stays_float32_and_agrees():
+    model, plain = setup("tiny-b", "float32", stored="float32")
+    lin = model.lm.layers[0].mixer.qkv
+    assert lin.weight.dtype == torch.float32 and model.lm.layers[0].norms["pre_mixer"].weight.dtype == torch.float32
+    mb, _ = setup("tiny-b", "bfloat16", stored="float32")
+    assert mb.lm.layers[0].mixer.qkv.weight.dtype == torch.float32                # not narrowed behind the user's back
+    toks = random_tokens(plain.V, 33, 14)
+    ref = plain.forward(toks)
+    for m, d in ((model, "float32"), (mb, "bfloat16")):
+        eng = m.engine(max_tokens=64)
+        s = eng.open(1)
+        assert max_err(eng.step(s, [toks], "all"), ref) < tol(d, ref)
+
+
+def test_step_argument_errors():
+    model, plain = setup("tiny-a", "float32")
+    eng = model.engine(max_tokens=128, max_seqs=2)
+    s = eng.open(2)
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.step(s, [[1], [256]])
+    with pytest.raises(ValueError, match="at least one token"):
+        eng.step(s, [[1], []])
+    with pytest.raises(alice.CacheError, match="full"):
+        eng.step(s, [[1] * 70, [2] * 70])
+    with pytest.raises(alice.CacheError, match="max_position"):
+        eng.step([s[0]], [[1] * 600])
+    assert eng.length(s[0]) == 0
+    with pytest.raises(alice.CacheError, match="all 2 slots"):
+        eng.open(1)
+    eng.close(s)

@@ -1,0 +1,309 @@
+"""Each kernel alone against a plain 64-bit reference of the same operation, at sizes other than the
+engine's, with inputs made so that a fault shows (a far key among hundreds, a window's edge, scattered
+pages)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from alice_llm_amd.hip import ops
+from plain import gemma2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+D = torch.float64
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, ref, atol, rtol=0.0):
+    err = (got.double().cpu() - ref.double().cpu()).abs()
+    bound = atol + rtol * ref.double().cpu().abs()
+    assert (err <= bound).all(), f"max err {err.max().item():.3e} (bound {bound.min().item():.1e}..)"
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("wdt", ["float32", "bfloat16"])
+def test_embed(wdt):
+    V, H = 301, 72
+    table = rnd(V, H, seed=1, dtype=DT[wdt])
+    tok = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, H, device=DEV)
+    ops.embed(tok, table, out, 3.25, V, H)
+    close(out, table.double()[tok.long()] * 3.25, 1e-6)
+
+
+# ------------------------------------------------------------------ residual add and norms
+@pytest.mark.parametrize("wdt,odt,full", [("float32", "float32", True), ("bfloat16", "bfloat16", False), ("bfloat16", "float32", True)])
+@pytest.mark.parametrize("H", [70, 2304, 5000])
+def test_add_norm_all_forms(wdt, odt, full, H):
+    T = 5
+    x0 = rnd(T, H, seed=2, scale=3.0)
+    br = rnd(3, T, H, seed=3, scale=0.5)
+    wp, wq = rnd(H, seed=4, scale=0.1, dtype=DT[wdt]), rnd(H, seed=5, scale=0.1, dtype=DT[wdt])
+    tol = 2e-6 if odt == "float32" else 2 ** -8
+    # pre norm only
+    out = torch.empty(T, H, dtype=DT[odt], device=DEV)
+    x = x0.clone()
+    ops.add_norm(x, None, None, wq, out, eps_pre=1e-5, off_pre=1.0, full_precision=full)
+    close(out, P.rms_norm(x0.double(), wq.double(), 1e-5), tol, tol)
+    assert torch.equal(x, x0)
+    # add of a post-normed sum of partials, then pre norm: one kernel
+    x = x0.clone()
+    ops.add_norm(x, br, wp, wq, out, eps_post=1e-6, eps_pre=1e-5, off_post=1.0, off_pre=0.0, n_partials=3, full_precision=full)
+    xr = x0.double() + P.rms_norm(br.double().sum(0), wp.double(), 1e-6)
+    close(x, xr, 1e-5)
+    close(out, P.rms_norm(xr, wq.double() - 1.0, 1e-5), tol * 4, tol)
+    # plain add (no post norm), no output
+    x = x0.clone()
+    ops.add_norm(x, br[0].contiguous(), None, None, None, full_precision=full)
+    close(x, x0.double() + br[0].double(), 1e-6)
+    # gathered rows
+    rows = torch.tensor([4, 0, 4], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, H, dtype=DT[odt], device=DEV)
+    ops.add_norm(x0.clone(), None, None, wq, out3, eps_pre=1e-5, off_pre=1.0, rows=rows, full_precision=full)
+    close(out3, P.rms_norm(x0.double()[rows.long()], wq.double(), 1e-5), tol, tol)
+
+
+def test_rms_norm_reference_vector_on_device():
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)                       # llama3.rs:20482-20498
+    out = torch.empty_like(x)
+    ops.add_norm(x, None, None, torch.zeros(4, device=DEV), out, eps_pre=1e-5, off_pre=1.0, full_precision=True)
+    close(out, x.double() / math.sqrt(7.5 + 1e-5), 1e-6)
+
+
+def test_softcap():
+    x = torch.tensor([-1e4, -50.0, -1.0, 0.0, 1e-3, 1.0, 29.0, 300.0, 1e30], device=DEV)
+    for full in (True, False):
+        y = x.clone()
+        ops.softcap_(y, 30.0, full)
+        close(y, 30.0 * torch.tanh(x.double() / 30.0), 1e-5 if full else 2e-4)
+
+
+# ------------------------------------------------------------------ matrix product
+LINEAR_SHAPES = [(1, 96, 64), (7, 200, 144), (64, 130, 320), (65, 64, 33), (300, 97, 100)]
+
+
+@pytest.mark.parametrize("M,N,K", LINEAR_SHAPES)
+@pytest.mark.parametrize("xdt,wdt,ydt", [("float32", "float32", "float32"), ("float32", "bfloat16", "float32"),
+                                          ("bfloat16", "bfloat16", "bfloat16"), ("bfloat16", "float32", "float32")])
+def test_linear_generic(M, N, K, xdt, wdt, ydt):
+    x, w = rnd(M, K, seed=6, dtype=DT[xdt]), rnd(N, K, seed=7, scale=0.1, dtype=DT[wdt])
+    y = torch.empty(M, N, dtype=DT[ydt], device=DEV)
+    full = xdt == "float32"
+    ops.linear(x, w, y, n_out=N, k_in=K, full_precision=full, variant=ops.LINEAR_GENERIC)
+    ref = x.double() @ w.double().T
+    close(y, ref, 1e-5 if ydt == "float32" else 1e-2, 0 if ydt == "float32" else 2 ** -8)
+    # softcap epilogue
+    y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(x, w, y2, n_out=N, k_in=K, epilogue=ops.EPI_SOFTCAP, epi_param=2.0, full_precision=full, variant=ops.LINEAR_GENERIC)
+    close(y2, 2.0 * torch.tanh(ref / 2.0), 1e-5 if full else 5e-4)
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 48, 64), (70, 160, 96), (9, 33, 40)])
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_linear_generic_geglu(M, N, K, dt):
+    x, w = rnd(M, K, seed=8, dtype=DT[dt]), rnd(2 * N, K, seed=9, scale=0.3, dtype=DT[dt])
+    y = torch.empty(M, N, dtype=DT[dt], device=DEV)
+    ops.linear(x, w, y, n_out=N, k_in=K, epilogue=ops.EPI_GEGLU, full_precision=dt == "float32", variant=ops.LINEAR_GENERIC)
+    g, u = x.double() @ w.double()[:N].T, x.double() @ w.double()[N:].T
+    # values reach about 20: the bound has an absolute part for the sums and a relative part for the product
+    close(y, F.gelu(g, approximate="tanh") * u, 2e-5 if dt == "float32" else 2e-2, 1e-5 if dt == "float32" else 2 ** -7)
+
+
+# ------------------------------------------------------------------ rotation and cache write
+def paged(T_max, nKV, d, dtype, n_seq, seed, page=64):
+    """Pools with more pages than needed and a scattered block table."""
+    per = -(-T_max // page)
+    n_pages = per * n_seq + 3
+    g = torch.Generator().manual_seed(seed)
+    perm = (torch.randperm(n_pages - 1, generator=g) + 1)[:per * n_seq].view(n_seq, per)
+    k = torch.zeros(n_pages, nKV, page, d, dtype=dtype, device=DEV)
+    return k, torch.zeros_like(k), perm.to(torch.int32).to(DEV)
+
+
+def fill_pools(kp, vp, bt, k, v, seq, start=0):
+    """k, v: [T, nKV, d] of sequence `seq`, written at positions start.."""
+    page = kp.shape[2]
+    for t in range(k.shape[0]):
+        p = int(bt[seq, (start + t) // page])
+        kp[p, :, (start + t) % page] = k[t].to(kp.dtype)
+        vp[p, :, (start + t) % page] = v[t].to(vp.dtype)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nH,nKV,d,R", [(4, 1, 16, 16), (6, 3, 24, 24), (2, 2, 40, 16), (3, 1, 256, 256)])
+def test_rope_cache_write(dt, nH, nKV, d, R):
+    lens, starts = [5, 70, 1], [0, 60, 130]
+    T = sum(lens)
+    qkv = rnd(T, (nH + 2 * nKV) * d + 8, seed=10, dtype=DT[dt])[:, :].contiguous()       # rows longer than the heads
+    pos = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    kp, vp, bt = paged(192, nKV, d, DT[dt], 3, seed=11)
+    theta = 5e5
+    j = torch.arange(R // 2, dtype=D)
+    ang = torch.arange(200, dtype=D)[:, None] * theta ** (-2.0 * j / R)
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    q_out = torch.empty(T, nH * d, dtype=DT[dt], device=DEV)
+    ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                         rotary_dim=R, max_position=int(pos.max()))
+    x = qkv.double().cpu()
+    q = x[:, :nH * d].view(T, nH, d)
+    k = x[:, nH * d:(nH + nKV) * d].view(T, nKV, d)
+    v = x[:, (nH + nKV) * d:(nH + 2 * nKV) * d].view(T, nKV, d)
+    def rot(a):
+        r = P.rope_half_split(a[..., :R], pos.cpu(), theta)
+        return torch.cat([r, a[..., R:]], dim=-1)
+    tol = 2e-6 if dt == "float32" else 2 ** -7
+    close(q_out.view(T, nH, d), rot(q), tol * 4, tol)
+    for t in range(T):
+        page, off = int(bt[int(seq[t]), int(pos[t]) // 64]), int(pos[t]) % 64
+        close(kp[page, :, off], rot(k)[t], tol * 4, tol)
+        close(vp[page, :, off], v[t], 0)
+    assert float(kp[0].abs().sum()) == 0 and int((kp.abs().sum(dim=(1, 3)) > 0).sum()) == T   # nothing else was touched
+    # q only, no cache
+    q2 = torch.empty_like(q_out)
+    ops.rope_cache_write(qkv, q2, None, None, cos, sin, pos, None, None, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                         rotary_dim=R, max_position=int(pos.max()))
+    assert torch.equal(q2, q_out)
+    with pytest.raises(ops.HipLibraryError, match="beyond the rotation tables"):
+        ops.rope_cache_write(qkv, q2, None, None, cos[:100], sin[:100], pos, None, None, num_heads=nH,
+                             num_kv_heads=nKV, head_dim=d, rotary_dim=R, max_position=int(pos.max()))
+
+
+# ------------------------------------------------------------------ attention
+def attention_case(dt, nH, nKV, d, lens, new, cap, window, seed, crafted=None):
+    """Sequences of total lengths `lens`, whose last `new[i]` tokens are the step's queries."""
+    B = len(lens)
+    kp, vp, bt = paged(max(lens), nKV, d, DT[dt], B, seed)
+    qs, refs, pos, seq = [], [], [], []
+    scale = 1.0 / math.sqrt(d * 1.7)
+    for b, (L, n) in enumerate(zip(lens, new)):
+        g = torch.Generator().manual_seed(seed * 100 + b)
+        q = torch.randn(L, nH, d, generator=g, dtype=D)
+        k = torch.randn(L, nKV, d, generator=g, dtype=D)
+        v = torch.randn(L, nKV, d, generator=g, dtype=D)
+        if crafted is not None:
+            crafted(b, q, k, v)
+        q, k, v = (t.to(DT[dt]).double() for t in (q, k, v))
+        fill_pools(kp, vp, bt, k, v, b)
+        refs.append(P.attention_core(q, k, v, scale, cap, window)[L - n:])
+        qs.append(q[L - n:])
+        pos += list(range(L - n, L))
+        seq += [b] * n
+    q = torch.cat(qs).reshape(-1, nH * d).to(DT[dt]).to(DEV)
+    return q, kp, vp, bt, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(seq, dtype=torch.int32, device=DEV), \
+        torch.cat(refs).reshape(-1, nH * d), scale
+
+
+ATT_SHAPES = [(4, 1, 16), (6, 3, 24), (8, 4, 64), (2, 1, 256), (5, 5, 40)]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nH,nKV,d", ATT_SHAPES)
+@pytest.mark.parametrize("cap,window", [(None, None), (5.0, 50), (50.0, 7)])
+def test_attention_generic_prompts_and_decode(dt, nH, nKV, d, cap, window):
+    for lens, new in (((5, 130, 66), (5, 130, 66)), ((200, 1, 77), (1, 1, 1)), ((150, 64), (20, 3))):
+        q, kp, vp, bt, pos, seq, ref, scale = attention_case(dt, nH, nKV, d, lens, new, cap, window, seed=3)
+        out = torch.empty_like(q)
+        ops.attention_generic(q, kp, vp, out, pos, seq, bt, num_heads=nH, scale=scale, softcap=cap, window=window,
+                              max_position=max(lens) - 1, full_precision=dt == "float32")
+        close(out, ref, 2e-5 if dt == "float32" else 2e-2)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_attention_far_key_and_window_edge(dt):
+    nH, nKV, d, L = 4, 2, 32, 700
+    # one far key (position 3) whose score towers over hundreds of others: the output is its value
+    def far(b, q, k, v):
+        k[3] = 0; k[3, :, 0] = 40.0
+        q[L - 1] = 0; q[L - 1, :, 0] = 40.0
+    q, kp, vp, bt, pos, seq, ref, scale = attention_case(dt, nH, nKV, d, (L,), (1,), None, None, seed=4, crafted=far)
+    out = torch.empty_like(q)
+    kw = dict(num_heads=nH, scale=scale, max_position=L - 1, full_precision=dt == "float32")
+    ops.attention_generic(q, kp, vp, out, pos, seq, bt, softcap=None, window=None, **kw)
+    close(out, ref, 2e-5 if dt == "float32" else 2e-2)
+    v3 = vp[int(bt[0, 0]), :, 3].double().cpu()
+    assert (out.view(nH, d)[0].double().cpu() - v3[0]).abs().max() < 1e-2
+    # a window of 100: the towering key at the first position outside (L - 101) is not seen, the one at the
+    # first position inside (L - 100) wins
+    for where, seen in ((L - 101, False), (L - 100, True)):
+        def edge(b, q, k, v, where=where):
+            k[where] = 0; k[where, :, 0] = 40.0; v[where] = 7.0
+            q[L - 1] = 0; q[L - 1, :, 0] = 40.0
+        q, kp, vp, bt, pos, seq, ref, scale = attention_case(dt, nH, nKV, d, (L,), (1,), None, 100, seed=5, crafted=edge)
+        out = torch.empty_like(q)
+        ops.attention_generic(q, kp, vp, out, pos, seq, bt, softcap=None, window=100, **kw)
+        close(out, ref, 2e-5 if dt == "float32" else 2e-2)
+        assert (abs(float(out[0, 0]) - 7.0) < 1e-2) == seen
+
+
+def test_attention_refuses_sizes_it_does_not_cover():
+    q, kp, vp, bt, pos, seq, ref, scale = attention_case("float32", 2, 1, 16, (9,), (9,), None, None, seed=6)
+    out = torch.empty_like(q)
+    with pytest.raises(ops.HipLibraryError, match="beyond the block table"):
+        ops.attention_generic(q, kp, vp, out, pos, seq, bt, num_heads=2, scale=scale, softcap=None, window=None,
+                              max_position=64, full_precision=True)
+    with pytest.raises(ops.HipLibraryError, match="head counts"):
+        ops.attention_generic(torch.empty(9, 48, device=DEV), kp.repeat(1, 2, 1, 1), vp.repeat(1, 2, 1, 1),
+                              torch.empty(9, 48, device=DEV), pos, seq, bt, num_heads=3, scale=scale, softcap=None,
+                              window=None, max_position=8, full_precision=True)
+    big = torch.zeros(2, 1, 64, 272, device=DEV)
+    with pytest.raises(ops.HipLibraryError, match="head_dim 272"):
+        ops.attention_generic(torch.empty(9, 272, device=DEV), big, big, torch.empty(9, 272, device=DEV), pos, seq, bt,
+                              num_heads=1, scale=scale, softcap=None, window=None, max_position=8, full_precision=True)
+
+
+# ------------------------------------------------------------------ sampling
+def test_argmax_lowest_index_on_ties():
+    x = rnd(5, 1000, seed=12)
+    x[1, 7] = x[1, 900] = 50.0
+    x[2] = 0.0
+    x[3, 999] = 60.0
+    got = ops.argmax(x).cpu().tolist()
+    assert got == [int(x[0].argmax()), 7, 0, 999, int(x[4].argmax())]
+    assert ops.argmax(torch.tensor([[0.7, 0.5, 0.7, 0.3]], device=DEV)).item() == 0    # llama3.rs:21263-21269
+
+
+def test_sample_reference_vectors():
+    probs = torch.tensor([[0.1, 0.2, 0.7]] * 3 + [[0.5, 0.5, 0.0]] * 3, device=DEV)     # integration_tests.rs
+    u = torch.tensor([0.05, 0.25, 0.95, 0.0, 0.49, 0.51], device=DEV)
+    assert ops.sample(probs.log(), u, 1.0).cpu().tolist() == [0, 1, 2, 0, 0, 1]
+    only = torch.tensor([[0.0, 0.0, 1.0, 0.0]], device=DEV).log()                        # llama3.rs:21390-21399
+    assert all(ops.sample(only, torch.tensor([x], device=DEV), 1.0).item() == 2 for x in (0.0, 0.5, 0.999999))
+
+
+@pytest.mark.parametrize("V", [384, 5000, 256000])
+def test_sample_matches_plain(V):
+    B = 6
+    logits = rnd(B, V, seed=13, scale=3.0)
+    g = torch.Generator().manual_seed(14)
+    for temperature, top_k, top_p in ((0.8, 0, 1.0), (1.5, 40, 1.0), (0.7, 0, 0.9), (1.0, 50, 0.5), (1e-3, 0, 1.0)):
+        u = torch.rand(B, generator=g)
+        got = ops.sample(logits, u.to(DEV), temperature, top_k, top_p).cpu().tolist()
+        for b in range(B):
+            want = P.plain_sample(logits[b].double().cpu(), temperature, top_k, top_p, float(u[b]))
+            if got[b] != want:
+                # a draw within rounding of a boundary of the cumulative sum may fall on either side
+                x = logits[b].double().cpu() / temperature
+                x = P.plain_top_p(P.plain_top_k(x, top_k), top_p)
+                cdf = torch.cumsum(P.plain_softmax(x), 0)
+                assert x[got[b]] > -math.inf and abs(float(cdf[min(got[b], want)]) - float(u[b])) < 1e-5, (b, got[b], want)
+
+
+def test_sample_frequencies():
+    logits = torch.tensor([[0.0, 0.0]], device=DEV).repeat(4000, 1)                       # llama3.rs:21401-21413
+    u = torch.rand(4000, generator=torch.Generator().manual_seed(15)).to(DEV)
+    ones = int(ops.sample(logits, u, 1.0).sum())
+    assert abs(ones - 2000) < 150
+    skew = torch.tensor([[0.0, 1.0, 2.0, 3.0]], device=DEV).repeat(4000, 1)
+    cold = ops.sample(skew, u, 0.01)
+    hot = ops.sample(skew, u, 1000.0)
+    assert int((cold == 3).sum()) == 4000 and 800 < int((hot == 0).sum()) < 1200          # llama3.rs:21339-21363
+    topk = ops.sample(skew, u, 1000.0, 2, 1.0)
+    assert set(topk.cpu().tolist()) == {2, 3}

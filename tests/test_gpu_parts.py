@@ -1,0 +1,324 @@
+"""Each part alone against its plain formula, built directly from its registry with sizes that no
+model here uses, and a toy architecture whose mixer keeps state of its own: registered, built,
+loaded with random weights and stepped without touching the package's files."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import alice_llm_amd as alice
+from alice_llm_amd.cache import Cache
+from alice_llm_amd.config.plan import LayerPlan, ModelPlan, PartSpec, ScheduleEntry
+from alice_llm_amd.engine.model import CausalLM
+from alice_llm_amd.engine.step import Engine
+from alice_llm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, CacheNeed, ParamSpec, Part, Precision,
+                                 ResidualStream, StateNeed)
+from alice_llm_amd.weights.loader import init_random
+from helpers import TOL
+from plain import gemma2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+D = torch.float64
+PRECS = ["float32", "bfloat16"]
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(prec):
+    return 2e-5 if prec == "float32" else 3e-2
+
+
+@pytest.mark.parametrize("prec", PRECS)
+def test_norm_part_and_stream_fusion(prec):
+    p = Precision.of(prec)
+    H, T = 136, 6
+    n1 = NORMS.get("rmsnorm")(p, dim=H, eps=3e-6, weight_offset=1.0)
+    n2 = NORMS.get("rmsnorm")(p, dim=H, eps=1e-5, weight_offset=0.0)
+    w1, w2 = rnd(H, seed=1, scale=0.1, dtype=torch.bfloat16), rnd(H, seed=2, dtype=torch.bfloat16)
+    n1.assign("weight", w1); n2.assign("weight", w2)
+    x0, br = rnd(T, H, seed=3, scale=2.0), rnd(T, H, seed=4)
+    s = ResidualStream(x0.clone(), p)
+    first = s.normed(n1)
+    assert first.dtype == p.act
+    ref_first = P.rms_norm(x0.double(), w1.double(), 3e-6)
+    assert (first.double() - ref_first).abs().max() < tol(prec)
+    s.push(br, n2)
+    second = s.normed(n1)                                      # add of the normed branch and the next norm, fused
+    xr = x0.double() + br.double() * torch.rsqrt((br.double() ** 2).mean(-1, keepdim=True) + 1e-5) * w2.double()
+    assert (s.x.double() - xr).abs().max() < 1e-5
+    assert (second.double() - P.rms_norm(xr, w1.double(), 3e-6)).abs().max() < tol(prec)
+    s.push(br, None)
+    rows = torch.tensor([5, 1], dtype=torch.int32, device=DEV)
+    last = s.rows_normed(n2, rows)
+    xr2 = xr + br.double()
+    want = xr2[[5, 1]] * torch.rsqrt((xr2[[5, 1]] ** 2).mean(-1, keepdim=True) + 1e-5) * w2.double()
+    assert (last.double() - want).abs().max() < tol(prec) * 4
+
+
+@pytest.mark.parametrize("prec", PRECS)
+def test_gated_mlp_part(prec):
+    p = Precision.of(prec)
+    H, I, T = 96, 208, 9
+    ff = FEED_FORWARDS.get("gated_mlp")(p, hidden_size=H, intermediate_size=I, activation="gelu_tanh")
+    assert {k: v.shape for k, v in ff.param_specs().items()} == {"gate_proj.weight": (I, H), "up_proj.weight": (I, H), "down_proj.weight": (H, I)}
+    ws = {n: rnd(*s.shape, seed=i, scale=0.2, dtype=torch.bfloat16) for i, (n, s) in enumerate(ff.param_specs().items())}
+    for n, w in ws.items():
+        ff.assign(n, w)
+    ff.finalize()
+    x = rnd(T, H, seed=9, dtype=p.act)
+    out = ff.forward(x, None)
+    out = out.sum(0) if out.dim() == 3 else out
+    ref = P.geglu(x.double(), ws["gate_proj.weight"].double(), ws["up_proj.weight"].double(), ws["down_proj.weight"].double())
+    assert out.dtype == torch.float32 and (out.double() - ref).abs().max() < tol(prec) * max(1.0, float(ref.abs().max()))
+    with pytest.raises(ValueError, match="activation"):
+        FEED_FORWARDS.get("gated_mlp")(p, hidden_size=H, intermediate_size=I, activation="relu6")
+
+
+@dataclass
+class _Ctx:
+    tokens: torch.Tensor
+    positions: torch.Tensor
+    seq_of_token: torch.Tensor
+    slots: torch.Tensor
+    max_position: int
+    is_decode: bool = False
+    want_rows: torch.Tensor = None
+    n_tokens: int = 0
+    n_seqs: int = 1
+    max_new: int = 0
+    max_context: int = 0
+    cu_seqlens: torch.Tensor = None
+    context_lens: torch.Tensor = None
+    new_lens: tuple = ()
+    start_lens: tuple = ()
+    slot_ids: tuple = ()
+
+
+def make_ctx(starts, news):
+    pos = [s + i for s, n in zip(starts, news) for i in range(n)]
+    seq = [b for b, n in enumerate(news) for _ in range(n)]
+    cu = [0]
+    for n in news:
+        cu.append(cu[-1] + n)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    return _Ctx(tokens=i32([0] * len(pos)), positions=i32(pos), seq_of_token=i32(seq), slots=i32(list(range(len(news)))),
+                max_position=max(pos), is_decode=all(n == 1 for n in news), n_tokens=len(pos), n_seqs=len(news),
+                max_new=max(news), max_context=max(s + n for s, n in zip(starts, news)), cu_seqlens=i32(cu),
+                context_lens=i32([s + n for s, n in zip(starts, news)]), new_lens=tuple(news), start_lens=tuple(starts),
+                slot_ids=tuple(range(len(news))))
+
+
+@pytest.mark.parametrize("prec", PRECS)
+@pytest.mark.parametrize("nH,nKV,d,window,cap,rotary", [(4, 2, 32, None, None, 32), (3, 1, 48, 20, 8.0, 48), (2, 2, 16, 70, 3.0, 8)])
+def test_attention_part_alone_in_two_steps(prec, nH, nKV, d, window, cap, rotary):
+    """The mixer on a cache of its own: a prompt step, then single tokens, against the plain formulas;
+    also a position encoding with a rotated width below the head size."""
+    p = Precision.of(prec)
+    H, T = 80, 90
+    rope = POSITIONS.get("rope")(p, DEV, dim=d, theta=3000.0, max_positions=128, rotary_dim=rotary)
+    att = MIXERS.get("attention")(p, {"r": rope}, hidden_size=H, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                                  scale=0.21, softcap=cap, window=window, position="r")
+    ws = {n: rnd(*s.shape, seed=10 + i, scale=0.15, dtype=torch.bfloat16) for i, (n, s) in enumerate(att.param_specs().items())}
+    for n, w in ws.items():
+        att.assign(n, w)
+    att.finalize()
+    need = att.cache_need()
+    assert need.kv.num_kv_heads == nKV and need.kv.head_dim == d and need.kv.window == window
+    cache = Cache([need], max_tokens=128, dtype=p.act, device=DEV, max_seqs=1)
+    slot = cache.open()
+    x = rnd(T, H, seed=20, dtype=p.act)
+    xd = x.double().cpu()
+    ws = {n: w.cpu() for n, w in ws.items()}
+    q = (xd @ ws["q_proj.weight"].double().T).view(T, nH, d)
+    k = (xd @ ws["k_proj.weight"].double().T).view(T, nKV, d)
+    v = (xd @ ws["v_proj.weight"].double().T).view(T, nKV, d)
+    pos = torch.arange(T)
+    rot = lambda a: torch.cat([P.rope_half_split(a[..., :rotary], pos, 3000.0), a[..., rotary:]], -1)
+    ref = P.attention_core(rot(q), rot(k), v, 0.21, cap, window).reshape(T, nH * d) @ ws["o_proj.weight"].double().T
+    got = []
+    for start, n in ((0, 70), (70, 1), (71, 1), (72, 18)):
+        cache.reserve([slot], [n])
+        bt = torch.tensor(cache.block_table_rows(0, [slot], 2), dtype=torch.int32, device=DEV)
+        out = att.forward(x[start:start + n].contiguous(), make_ctx([start], [n]), cache.view(0, [bt]))
+        got.append(out.sum(0) if out.dim() == 3 else out)
+        cache.commit([slot], [n])
+    got = torch.cat(got)
+    assert (got.double().cpu() - ref.cpu()).abs().max() < tol(prec) * max(1.0, float(ref.abs().max()))
+
+
+# ------------------------------------------------------------------ a toy architecture
+class ToyDecayMixer(Part):
+    """A mixer with state of its own and no keys: s <- a * s + x W_in per token, output s W_out.  State is a
+    fixed-size vector per sequence, advanced token by token inside a step (a sequential scan in torch: this
+    is a test of the interfaces, not a kernel)."""
+
+    def __init__(self, precision, positions, *, hidden_size, state_size, decay):
+        self.p, self.H, self.S, self.decay = precision, hidden_size, state_size, decay
+        self.w = {}
+
+    def param_specs(self):
+        return {"in.weight": ParamSpec((self.S, self.H), 0.1), "out.weight": ParamSpec((self.H, self.S), 0.1)}
+
+    def assign(self, name, t):
+        self.w[name] = t.float()
+
+    def cache_need(self):
+        return CacheNeed(state=StateNeed((self.S,), torch.float32))
+
+    def forward(self, x, ctx, cache):
+        u = x.float() @ self.w["in.weight"].T
+        out = torch.empty_like(u)
+        row = 0
+        for slot, n in zip(ctx.slot_ids, ctx.new_lens):
+            s = cache.state[slot]
+            for i in range(n):
+                s = self.decay * s + u[row]
+                out[row] = s
+                row += 1
+            cache.state[slot] = s
+        return (out @ self.w["out.weight"].T).contiguous()
+
+
+class ToyMLP(Part):
+    def __init__(self, precision, *, hidden_size):
+        self.H = hidden_size
+
+    def param_specs(self):
+        return {"w.weight": ParamSpec((self.H, self.H), 0.1)}
+
+    def assign(self, name, t):
+        self.w = t.float()
+
+    def forward(self, x, ctx):
+        return torch.relu(x.float() @ self.w.T).contiguous()
+
+
+class ToyConfig:
+    def __init__(self, d):
+        self.d = dict(d)
+        self.torch_dtype = "bfloat16"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def plan(self):
+        H, V, L = self.d["width"], self.d["vocab"], self.d["depth"]
+        norm = lambda name: PartSpec("rmsnorm", {"dim": H, "eps": 1e-5, "weight_offset": 0.0}, name)
+        layers = []
+        for i in range(L):
+            toy = i % 2 == 0      # toy mixer on even layers, windowed attention on odd ones: one model, two mixers
+            mixer = (PartSpec("toy_decay", {"hidden_size": H, "state_size": self.d["state"], "decay": 0.5}, "mix") if toy else
+                     PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "scale": 0.25,
+                                            "window": 5, "position": "rope"}, "attn"))
+            layers.append(LayerPlan(block="prenorm", mixer=mixer, feed_forward=PartSpec("toy_mlp", {"hidden_size": H}, "ff"),
+                                    norms={"pre_mixer": norm("n1"), "pre_ff": norm("n2")}, prefix=f"blocks.{i}."))
+        # the schedule runs layer 0 twice (each run with state of its own), and layer 3 reads the cache that
+        # the run of layer 1 (entry 1) wrote
+        schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(2), ScheduleEntry(3, cache_from=1)]
+        return ModelPlan(vocab_size=V, hidden_size=H, max_positions=256,
+                         embedding=PartSpec("embedding", {"vocab_size": V, "dim": H, "scale": 1.0}, "emb"),
+                         positions={"rope": PartSpec("rope", {"dim": 16, "theta": 100.0, "max_positions": 256})},
+                         layers=tuple(layers), schedule=tuple(schedule[:L + 1] if L >= 4 else schedule[:3]),
+                         final_norm=norm("final"), head=PartSpec("lm_head", {"vocab_size": V, "dim": H, "tied_to": "emb"}, "head"))
+
+
+def toy_plain(model, tokens):
+    """The toy model for one whole sequence in 64-bit, from the loaded tensors."""
+    lm = model.lm
+    get = lambda part: part.weight.double().cpu() if hasattr(part, "weight") else None
+    E = lm.embedding.table.weight.double().cpu()
+    x = E[torch.tensor(tokens)]
+    T = len(tokens)
+    rms = lambda v, n: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + n.eps) * (n.weight_offset + n.weight.double().cpu())
+    kv_seen = {}
+    for ei, e in enumerate(lm.plan.schedule):
+        layer = lm.layers[e.layer]
+        h = rms(x, layer.norms["pre_mixer"])
+        m = layer.mixer
+        if isinstance(m, ToyDecayMixer):
+            u = h @ m.w["in.weight"].double().cpu().T
+            s = torch.zeros(m.S, dtype=D)           # every run of the schedule has state of its own
+            outs = []
+            for i in range(T):
+                s = 0.5 * s + u[i]
+                outs.append(s)
+            a = torch.stack(outs) @ m.w["out.weight"].double().cpu().T
+        else:
+            W = m.qkv.weight.double().cpu()
+            q = (h @ W[:32].T).view(T, 2, 16)
+            if e.cache_from is None:
+                k = P.rope_half_split((h @ W[32:48].T).view(T, 1, 16), torch.arange(T), 100.0)
+                v = (h @ W[48:64].T).view(T, 1, 16)
+                kv_seen[ei] = (k, v)
+            else:
+                k, v = kv_seen[e.cache_from]
+            o = P.attention_core(P.rope_half_split(q, torch.arange(T), 100.0), k, v, 0.25, None, 5)
+            a = o.reshape(T, 32) @ m.o.weight.double().cpu().T
+        x = x + a
+        h = rms(x, layer.norms["pre_ff"])
+        x = x + torch.relu(h @ layer.feed_forward.w.double().cpu().T)
+    return rms(x, lm.final_norm) @ E.T
+
+
+def test_toy_architecture_with_a_stateful_mixer_registers_builds_and_steps():
+    MIXERS.register("toy_decay", ToyDecayMixer)
+    FEED_FORWARDS.register("toy_mlp", ToyMLP)
+    alice.register_architecture("ToyForCausalLM", ToyConfig)
+    raw = {"architectures": ["ToyForCausalLM"], "width": 48, "vocab": 77, "depth": 4, "state": 24}
+    assert "ToyForCausalLM" in alice.registered_architectures()
+    # float32 weights stay row-major, which the toy's 64-bit replica reads directly
+    model = alice.Model.random(raw, seed=3, dtype="float32", stored_dtype=torch.float32)
+    assert list(model.lm.param_specs())[:3] == ["emb.weight", "blocks.0.mix.in.weight", "blocks.0.mix.out.weight"]
+    eng = model.engine(max_tokens=256, max_seqs=3)
+    assert [g.layers for g in eng.cache.groups] == [[1]] and sorted(eng.cache.state) == [0, 2, 3]   # by schedule entry
+    seqs = [[5, 9, 3, 70, 1, 22, 8, 8, 41, 60, 2, 13], [7, 7, 30], [11, 2, 64, 19, 50, 6]]
+    # cut-up runs of the engine against its own whole runs, and both against the 64-bit replica
+    slots = eng.open(3)
+    whole = eng.step(slots, seqs, "all")
+    eng.close(slots)
+    slots = eng.open(3)
+    parts = [eng.step(slots, [s[:2] for s in seqs], "all")]
+    left = [s[2:] for s in seqs]
+    live = [0, 1, 2]
+    outs = {i: [] for i in live}
+    while live:
+        lg = eng.step([slots[i] for i in live], [[left[i].pop(0)] for i in live], "last")
+        for row, i in enumerate(live):
+            outs[i].append(lg[row])
+        done = [i for i in live if not left[i]]
+        eng.close([slots[i] for i in done])                    # state of a closed slot is zeroed when it is taken again
+        live = [i for i in live if i not in done]
+    first = parts[0]
+    cut = torch.cat([torch.cat([first[2 * i:2 * i + 2], torch.stack(outs[i])]) for i in range(3)])
+    assert (cut - whole).abs().max() < 1e-5
+    ref = torch.cat([toy_plain(model, t) for t in seqs])
+    assert (whole.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
+    # slots used again start from zero state: the same requests give the same logits
+    slots = eng.open(3)
+    assert torch.equal(eng.step(slots, seqs, "all"), whole)
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
+def test_toy_architecture_against_its_plain_replica():
+    MIXERS.register("toy_decay", ToyDecayMixer)
+    FEED_FORWARDS.register("toy_mlp", ToyMLP)
+    alice.register_architecture("ToyForCausalLM", ToyConfig)
+    raw = {"architectures": ["ToyForCausalLM"], "width": 48, "vocab": 77, "depth": 4, "state": 24}
+    model = alice.Model.random(raw, seed=4, dtype="float32", stored_dtype=torch.float32)
+    eng = model.engine(max_tokens=128, max_seqs=2)
+    toks = [5, 9, 3, 70, 1, 22, 8, 8, 41, 60, 2, 13, 0, 76]
+    s = eng.open(1)
+    got = torch.cat([eng.step(s, [toks[:9]], "all")] + [eng.step(s, [[t]], "last") for t in toks[9:]])
+    ref = toy_plain(model, toks)
+    assert (got.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
