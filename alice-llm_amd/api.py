@@ -39,8 +39,10 @@ class Model:
         return cls(config, lm)
 
     @classmethod
-    def random(cls, config, seed: int = 0, dtype=None, device=None, stored_dtype: Optional[torch.dtype] = None) -> "Model":
-        """Random weights straight onto the device: the same tensors write_random_model(config, seed) writes."""
+    def random(cls, config, seed: int = 0, dtype=None, device=None, stored_dtype: Optional[torch.dtype] = None,
+               fast: bool = False) -> "Model":
+        """Random weights straight onto the device: the same tensors write_random_model(config, seed) writes
+        (with fast=True they are drawn on the GPU instead: same distribution, other values)."""
         if isinstance(config, dict):
             config = config_from_dict(config)
         device = torch.device(device) if device is not None else ops.require_gpu()
@@ -48,7 +50,7 @@ class Model:
         lm = CausalLM(config.plan(), precision, device)
         if stored_dtype is None:
             stored_dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[getattr(config, "torch_dtype", "bfloat16")]
-        init_random(lm, seed, stored_dtype)
+        init_random(lm, seed, stored_dtype, on_device=fast)
         return cls(config, lm)
 
     # ------------------------------------------------------------------ use

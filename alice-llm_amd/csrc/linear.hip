@@ -2,9 +2,12 @@
 #include "common.h"
 #include "alice_hip.h"
 
+int alice_linear_split_hint_frag(int M, int N, int K);
+int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_dtype, int M, int N, int K,
+                      int epi, float epi_param, int split_k, int variant, hipStream_t stream);
+
 extern "C" int alice_linear_split_hint(int M, int N, int K, int w_layout) {
-  (void)M; (void)N; (void)K; (void)w_layout;
-  return 1;
+  return w_layout == ALICE_LAYOUT_FRAG16 ? alice_linear_split_hint_frag(M, N, K) : 1;
 }
 
 extern "C" int alice_linear(const void* x, int x_dtype, const void* w, int w_dtype, int w_layout, void* y,
@@ -19,12 +22,11 @@ extern "C" int alice_linear(const void* x, int x_dtype, const void* w, int w_dty
     return alice_linear_generic(x, x_dtype, w, w_dtype, y, y_dtype, M, N, K, epilogue, epi_param,
                                 full_precision, stream);
   }
+  if (w_layout == ALICE_LAYOUT_FRAG16) {
+    ALICE_CHECK(w_dtype == DT_BF16, "linear: the fragment layout holds bfloat16 only");
+    ALICE_CHECK(variant != ALICE_LINEAR_GENERIC, "linear: the generic kernel reads row-major weights");
+    return alice_linear_frag(x, x_dtype, w, y, y_dtype, M, N, K, epilogue, epi_param, split_k, variant, stream);
+  }
   alice_set_error("linear: unknown weight layout %d", w_layout);
-  return 1;
-}
-
-extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream) {
-  (void)src; (void)dst; (void)N; (void)K; (void)stream;
-  alice_set_error("to_frag16: not built");
   return 1;
 }

@@ -1,0 +1,377 @@
+// bfloat16 matrix products on the matrix cores (MFMA 16x16x32, 32-bit accumulation), reading
+// weights in a fragment layout that is made once at load.
+//
+// Fragment layout of W[N, K] (bfloat16): tiles of 16 rows x 32 columns, stored tile by tile as
+// [N/16][K/32][64 lanes][8 elements]; lane l = g*16 + r of a tile holds W[n0 + r][k0 + 8g .. 8g+7],
+// which is exactly what lane l supplies to the MFMA as its part of the 16x32 operand.  A wave
+// therefore loads a whole tile with one fully coalesced 1 KB read and no shuffle through LDS.
+// N is padded to a multiple of 16 and K to a multiple of 32 with zeros.
+//
+// Operand roles: the weight tile is the MFMA's first operand (rows = output features n), the
+// activations the second (columns = tokens m).  Lane l then holds D[n = 4*(l/16) + i][m = l%16],
+// i = 0..3: four consecutive output features of one token, stored with one vector store.
+//
+// Two kernels share this: a weight-streaming kernel for up to 64 tokens (decode), whose four waves
+// split the inner dimension and add their parts in a fixed order, and a tiled kernel for many
+// tokens (prompts).  The math is the reference's y[r] = sum_c W[r,c] x[c] (gguf.rs:4063-4074) with the
+// GeGLU (llama3.rs:14519-14534) and softcap (llama3.rs:14606-14611) epilogues.
+#include "common.h"
+#include "alice_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
+}
+
+// The activation fragment of token row `m` (clamped by the caller) at k-tile kt: 8 consecutive elements.
+__device__ __forceinline__ u32x4 load_x_frag(const bf16_t* __restrict__ x, int row, bool row_ok, int K, int kt, int g) {
+  const int k = kt * 32 + g * 8;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (row_ok && k < K) v = *reinterpret_cast<const u32x4*>(x + (size_t)row * K + k);
+  return v;
+}
+
+template <int EPI, bool FULL>
+__device__ __forceinline__ float epilogue1(float v, float p) {
+  if (EPI == ALICE_EPI_SOFTCAP) return p * (FULL ? tanh_full(v / p) : tanh_fast(v / p));
+  return v;
+}
+
+template <typename TO>
+__device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n, int N, f32x4 v) {
+  if (n + 3 < N && (((size_t)row_off + n) & 3) == 0) {
+    if constexpr (sizeof(TO) == 4) {
+      *reinterpret_cast<f32x4*>((float*)y + row_off + n) = v;
+    } else {
+      uint32_t lo = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+      uint32_t hi = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+      uint2 pk = {lo, hi};
+      *reinterpret_cast<uint2*>((bf16_t*)y + row_off + n) = pk;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) store_f32(y, row_off + n + i, v[i]);
+  }
+}
+
+// ---------------------------------------------------------------- weight streaming, M <= 16*MT
+// Block: 4 waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + 4, ...; the parts of
+// waves 1..3 go through LDS and wave 0 adds them in the order 1, 2, 3.  grid.x: groups of RT row
+// tiles (for GeGLU: RT/2 gate tiles and the RT/2 up tiles that belong to them); grid.y: slices of the
+// inner dimension, each writing its own partial sum y[slice][M][N] (slices > 1 only without epilogue).
+template <int RT, int MT, int EPI, typename TO, bool FULL>
+__global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+                                                            TO* __restrict__ y, int M, int N, int K, int KT, int NT,
+                                                            int kt_per_slice, float epi) {
+  extern __shared__ __align__(16) float red[];            // [3][RT*MT][64][4]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int kb = blockIdx.y * kt_per_slice, ke = min(KT, kb + kt_per_slice);
+
+  int tile[RT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i) {
+    if (EPI == ALICE_EPI_GEGLU) tile[i] = (i & 1) ? (N / 16 + blockIdx.x * (RT / 2) + (i >> 1)) : (blockIdx.x * (RT / 2) + (i >> 1));
+    else tile[i] = blockIdx.x * RT + i;
+  }
+  const int tile_limit = NT;
+  f32x4 acc[RT][MT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  bool row_ok[MT];
+  int row[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) { row[j] = j * 16 + r; row_ok[j] = row[j] < M; }
+
+  constexpr int U = RT >= 4 ? 2 : 4;                      // k-tiles in flight per wave
+  for (int kt0 = kb + wave * U; kt0 < ke; kt0 += 4 * U) {
+    u32x4 a[U][RT], b[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = kt0 + u;
+      const bool kok = kt < ke;
+#pragma unroll
+      for (int i = 0; i < RT; ++i) {
+        a[u][i] = u32x4{0u, 0u, 0u, 0u};
+        if (kok && tile[i] < tile_limit)
+          a[u][i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j) b[u][j] = load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[i][j] = mfma16(a[u][i], b[u][j], acc[i][j]);
+  }
+
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        *reinterpret_cast<f32x4*>(red + ((size_t)((wave - 1) * RT * MT + i * MT + j) * 64 + lane) * 4) = acc[i][j];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w)
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        f32x4 p = *reinterpret_cast<const f32x4*>(red + ((size_t)(w * RT * MT + i * MT + j) * 64 + lane) * 4);
+        acc[i][j] += p;
+      }
+
+  TO* yo = y + (size_t)blockIdx.y * M * N;                // the slice's partial sum
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    if (!row_ok[j]) continue;
+    const size_t row_off = (size_t)row[j] * N;
+    if (EPI == ALICE_EPI_GEGLU) {
+#pragma unroll
+      for (int p = 0; p < RT / 2; ++p) {
+        const int n = (blockIdx.x * (RT / 2) + p) * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = gelu_tanh_f(acc[2 * p][j][i], FULL) * acc[2 * p + 1][j][i];
+        store4(yo, row_off, n, N, o);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < RT; ++i) {
+        const int n = tile[i] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
+        store4(yo, row_off, n, N, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- tiled, many tokens
+// Block: 4 waves side by side along N; every wave computes 128 tokens x 64 output features
+// (8 x 4 MFMA tiles, 128 accumulator registers per lane) and streams its own weight tiles; the four
+// waves read the same activation rows (through the vector cache).  grid.x: groups of 16 row tiles
+// (256 features; for GeGLU 128 output features = 8 gate + 8 up tiles); grid.y: groups of 128 tokens.
+constexpr int WM = 8, WN = 4;
+
+template <int EPI, typename TO, bool FULL>
+__global__ __launch_bounds__(256) void linear_tiled_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
+                                                                float epi) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int m0 = blockIdx.y * (16 * WM);
+  int tile[WN];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) {
+    if (EPI == ALICE_EPI_GEGLU) {
+      const int pair = (blockIdx.x * 4 + wave) * (WN / 2) + (i >> 1);
+      tile[i] = (i & 1) ? N / 16 + pair : pair;
+      if (pair >= N / 16) tile[i] = NT;                    // beyond the matrix
+    } else {
+      tile[i] = (blockIdx.x * 4 + wave) * WN + i;
+    }
+  }
+  int row[WM];
+#pragma unroll
+  for (int j = 0; j < WM; ++j) row[j] = min(m0 + j * 16 + r, M - 1);      // clamped: extra rows are computed and dropped
+
+  f32x4 acc[WN][WM];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 a[WN], b[WM], an[WN], bn[WM];
+  auto load_tile = [&](int kt, u32x4* aa, u32x4* bb) {
+#pragma unroll
+    for (int i = 0; i < WN; ++i) {
+      aa[i] = u32x4{0u, 0u, 0u, 0u};
+      if (tile[i] < NT) aa[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < WM; ++j) bb[j] = load_x_frag(x, row[j], true, K, kt, g);
+  };
+  load_tile(0, a, b);
+  for (int kt = 0; kt < KT; ++kt) {
+    if (kt + 1 < KT) load_tile(kt + 1, an, bn);
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
+#pragma unroll
+    for (int i = 0; i < WN; ++i) a[i] = an[i];
+#pragma unroll
+    for (int j = 0; j < WM; ++j) b[j] = bn[j];
+  }
+
+#pragma unroll
+  for (int j = 0; j < WM; ++j) {
+    const int m = m0 + j * 16 + r;
+    if (m >= M) continue;
+    const size_t row_off = (size_t)m * N;
+    if (EPI == ALICE_EPI_GEGLU) {
+#pragma unroll
+      for (int p = 0; p < WN / 2; ++p) {
+        if (tile[2 * p] >= NT) continue;
+        const int n = tile[2 * p] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
+        store4(y, row_off, n, N, o);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < WN; ++i) {
+        if (tile[i] >= NT) continue;
+        const int n = tile[i] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
+        store4(y, row_off, n, N, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- layout conversion
+__global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N, int K, int KT, size_t total) {
+  const size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x;     // index in dst, in elements
+  if (o >= total) return;
+  const int e = o & 7;
+  const int lane = (o >> 3) & 63;
+  const size_t t = o >> 9;
+  const int kt = (int)(t % KT);
+  const int nt = (int)(t / KT);
+  const int n = nt * 16 + (lane & 15), k = kt * 32 + (lane >> 4) * 8 + e;
+  bf16_t z;
+  z.bits = 0;
+  dst[o] = (n < N && k < K) ? src[(size_t)n * K + k] : z;
+}
+
+template <int RT, int MT, int EPI, typename TO>
+int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
+  const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
+  const int groups = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, RT / 2) : ceil_div(NT, RT);
+  const int per = ceil_div(KT, split);
+  dim3 grid(groups, split);
+  const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
+  linear_skinny_kernel<RT, MT, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
+// Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
+// on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)
+int skinny_row_tiles(int N, int epi) {
+  const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
+  if (tiles >= 4096) return 4;
+  if (tiles >= 1024 || epi == ALICE_EPI_GEGLU) return 2;
+  return 1;
+}
+
+template <int EPI, typename TO>
+int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
+  const int rt = skinny_row_tiles(N, EPI);
+#define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, s)
+#define BY_RT(MT)                                                   \
+  do {                                                              \
+    if (rt == 4) GO(4, MT);                                         \
+    if (rt == 2) GO(2, MT);                                         \
+    if constexpr (EPI != ALICE_EPI_GEGLU) GO(1, MT);                \
+  } while (0)
+  if (M <= 16) BY_RT(1);
+  if (M <= 32) BY_RT(2);
+  BY_RT(4);
+#undef BY_RT
+#undef GO
+  return 1;
+}
+
+template <int EPI, typename TO>
+int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, float epi, hipStream_t s) {
+  const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
+  const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
+  dim3 grid(gx, ceil_div(M, 16 * WM));
+  linear_tiled_mfma_kernel<EPI, TO, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int alice_has_mfma_linear() { return 1; }
+
+// Whether a matrix of `rows` x K with this epilogue can use the fragment layout.
+extern "C" int alice_frag16_supported(int rows, int K, int epilogue) {
+  if (K % 8 != 0) return 0;                                   // activations are read 8 at a time
+  if (epilogue == ALICE_EPI_GEGLU && (rows % 32 != 0)) return 0;   // gate and up halves must be whole tiles
+  return 1;
+}
+
+extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream) {
+  ALICE_CHECK(N > 0 && K > 0, "to_frag16: bad sizes N=%d K=%d", N, K);
+  const int KT = (K + 31) / 32, NT = (N + 15) / 16;
+  const size_t total = (size_t)NT * KT * 512;
+  to_frag16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>((const bf16_t*)src, (bf16_t*)dst, N, K, KT, total);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
+int alice_linear_split_hint_frag(int M, int N, int K) {
+  if (M > 64) return 1;
+  const int KT = (K + 31) / 32;
+  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(N, ALICE_EPI_NONE));
+  int split = 1;
+  // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
+  while (groups * split < 1024 && KT / (split * 2) >= 16 && split < 16) split *= 2;
+  return split;
+}
+
+int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_dtype, int M, int N, int K,
+                      int epi, float epi_param, int split_k, int variant, hipStream_t stream) {
+  ALICE_CHECK(x_dtype == DT_BF16, "linear: the fragment layout needs bfloat16 activations");
+  ALICE_CHECK(dtype_ok(y_dtype), "linear: unknown output dtype");
+  ALICE_CHECK(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear: bad sizes M=%d N=%d K=%d (K must be a multiple of 8)", M, N, K);
+  ALICE_CHECK(epi != ALICE_EPI_GEGLU || N % 16 == 0, "linear: GeGLU in the fragment layout needs N %% 16 == 0, found %d", N);
+  ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f, "linear: softcap must be positive");
+  ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0, "linear: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64);
+  ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
+  ALICE_CHECK(split_k == 1 || (skinny && epi == ALICE_EPI_NONE && y_dtype == DT_F32),
+              "linear: partial sums need the streaming kernel, no epilogue and float32 output");
+  ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
+#define BY_EPI(FN, ...)                                                                            \
+  do {                                                                                             \
+    if (y_dtype == DT_F32) {                                                                       \
+      if (epi == ALICE_EPI_NONE) return FN<ALICE_EPI_NONE, float>(__VA_ARGS__);                    \
+      if (epi == ALICE_EPI_GEGLU) return FN<ALICE_EPI_GEGLU, float>(__VA_ARGS__);                  \
+      return FN<ALICE_EPI_SOFTCAP, float>(__VA_ARGS__);                                            \
+    } else {                                                                                       \
+      if (epi == ALICE_EPI_NONE) return FN<ALICE_EPI_NONE, bf16_t>(__VA_ARGS__);                   \
+      if (epi == ALICE_EPI_GEGLU) return FN<ALICE_EPI_GEGLU, bf16_t>(__VA_ARGS__);                 \
+      return FN<ALICE_EPI_SOFTCAP, bf16_t>(__VA_ARGS__);                                           \
+    }                                                                                              \
+  } while (0)
+  if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, stream);
+  BY_EPI(launch_tiled, x, w, y, M, N, K, epi_param, stream);
+#undef BY_EPI
+}

@@ -41,6 +41,7 @@ def _declare(lib) -> None:
         "alice_linear": [P, I, P, I, I, P, I, I, I, I, I, F, I, I, I, P],
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
+        "alice_frag16_supported": [I, I, I],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, I, I, P],
@@ -293,9 +294,9 @@ def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
           float(softcap or 0.0), int(window or 0), int(full_precision), _stream())
 
 
-def fragment_layout_available() -> bool:
-    """Whether this build of the library has the MFMA kernels that read the fragment layout."""
-    return bool(getattr(library(), "alice_has_mfma_linear", lambda: 0)())
+def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
+    """Whether the MFMA kernels take a weight of `rows` x k_in with this epilogue in the fragment layout."""
+    return bool(library().alice_frag16_supported(int(rows), int(k_in), int(epilogue)))
 
 
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,

@@ -39,7 +39,7 @@ class Linear:
         if tuple(w.shape) != (self.weight_rows, self.k):
             raise ValueError(f"weight must be {(self.weight_rows, self.k)}, found {tuple(w.shape)}")
         if (USE_FRAGMENT_LAYOUT and self.precision.name == "bfloat16" and w.dtype == torch.bfloat16
-                and ops.fragment_layout_available()):
+                and ops.fragment_layout_supported(self.weight_rows, self.k, self.epilogue)):
             self.weight = ops.to_frag16(w.contiguous())
             self.layout = ops.LAYOUT_FRAG16
         else:

@@ -78,25 +78,27 @@ def load_weights(model, folder: str) -> None:
 
 # --------------------------------------------------------------------------- random weights
 
-def random_tensors(specs: Dict[str, ParamSpec], seed: int, dtype: torch.dtype) -> Iterator[Tuple[str, torch.Tensor]]:
+def random_tensors(specs: Dict[str, ParamSpec], seed: int, dtype: torch.dtype, device="cpu") -> Iterator[Tuple[str, torch.Tensor]]:
     """Tensors in the order of `specs` from one generator seeded with `seed`: N(0, init_std) drawn in
-    float32 on the host, then cast to `dtype`; integer tables are zeros."""
-    gen = torch.Generator(device="cpu")
+    float32 (on the host unless a device is given, whose generator draws other values), then cast to
+    `dtype`; integer tables are zeros."""
+    gen = torch.Generator(device=device)
     gen.manual_seed(int(seed))
     for name, spec in specs.items():
         if spec.integer:
-            yield name, torch.zeros(spec.shape, dtype=torch.int32)
+            yield name, torch.zeros(spec.shape, dtype=torch.int32, device=device)
         else:
-            t = torch.empty(spec.shape, dtype=torch.float32)
+            t = torch.empty(spec.shape, dtype=torch.float32, device=device)
             t.normal_(0.0, spec.init_std, generator=gen)
             yield name, t.to(dtype)
 
 
-def init_random(model, seed: int, dtype: Optional[torch.dtype] = None) -> None:
-    """Fill the model with the tensors that `write_random_model` would write for the same seed."""
+def init_random(model, seed: int, dtype: Optional[torch.dtype] = None, on_device: bool = False) -> None:
+    """Fill the model with the tensors that `write_random_model` would write for the same seed
+    (on_device: drawn by the GPU's generator instead, for large models where only the distribution matters)."""
     dtype = dtype or torch.bfloat16
     specs = model.param_specs()
-    for name, t in random_tensors(specs, seed, dtype):
+    for name, t in random_tensors(specs, seed, dtype, model.device if on_device else "cpu"):
         _place(model, name, specs[name], t)
     model.finalize()
 

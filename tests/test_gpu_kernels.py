@@ -307,3 +307,84 @@ def test_sample_frequencies():
     assert int((cold == 3).sum()) == 4000 and 800 < int((hot == 0).sum()) < 1200          # llama3.rs:21339-21363
     topk = ops.sample(skew, u, 1000.0, 2, 1.0)
     assert set(topk.cpu().tolist()) == {2, 3}
+
+
+# ------------------------------------------------------------------ matrix-core matrix products
+def frag_reference(w):
+    """The fragment layout written out in plain indexing: [N/16][K/32][lane = g*16 + r][8]."""
+    N, K = w.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 32) * 32
+    wp = torch.zeros(Np, Kp, dtype=w.dtype)
+    wp[:N, :K] = w.cpu()
+    return wp.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+
+
+def test_fragment_layout():
+    for N, K in ((16, 32), (40, 72), (96, 64), (33, 8)):
+        w = rnd(N, K, seed=N, dtype=torch.bfloat16)
+        assert torch.equal(ops.to_frag16(w).cpu(), frag_reference(w))
+    assert ops.fragment_layout_supported(96, 64, ops.EPI_NONE) and not ops.fragment_layout_supported(96, 36, ops.EPI_NONE)
+    assert ops.fragment_layout_supported(64, 64, ops.EPI_GEGLU) and not ops.fragment_layout_supported(48, 64, ops.EPI_GEGLU)
+
+
+MFMA_SHAPES = [(1, 96, 64), (7, 208, 144), (16, 4096, 256), (17, 130, 320), (33, 64, 96), (64, 2304, 1024),
+               (65, 304, 160), (128, 256, 64), (300, 1000, 416), (1000, 80, 2048)]
+
+
+@pytest.mark.parametrize("M,N,K", MFMA_SHAPES)
+@pytest.mark.parametrize("ydt", ["float32", "bfloat16"])
+def test_linear_mfma(M, N, K, ydt):
+    x, w = rnd(M, K, seed=16, dtype=torch.bfloat16), rnd(N, K, seed=17, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    ref = x.double() @ w.double().T
+    atol, rtol = (2e-4, 1e-5) if ydt == "float32" else (1e-2, 2 ** -8)
+    variants = [ops.LINEAR_MFMA] + ([ops.LINEAR_SKINNY] if M <= 64 else [])
+    for variant in variants:
+        y = torch.full((M, N), float("nan"), dtype=DT[ydt], device=DEV)
+        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=variant, full_precision=False)
+        close(y, ref, atol * math.sqrt(K / 64), rtol)
+        y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        ops.linear(x, wf, y2, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_SOFTCAP, epi_param=3.0,
+                   variant=variant, full_precision=False)
+        close(y2, 3.0 * torch.tanh(ref / 3.0), 1e-3)
+    if M <= 64:
+        for split in (2, 3, 8):
+            yp = torch.full((split, M, N), float("nan"), dtype=torch.float32, device=DEV)
+            ops.linear(x, wf, yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=ops.LINEAR_SKINNY,
+                       full_precision=False)
+            close(yp.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 48, 96), (200, 304, 96), (129, 2048, 64)])
+def test_linear_mfma_geglu(M, N, K):
+    x, w = rnd(M, K, seed=18, dtype=torch.bfloat16), rnd(2 * N, K, seed=19, scale=0.3, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    g, u = x.double() @ w.double()[:N].T, x.double() @ w.double()[N:].T
+    ref = F.gelu(g, approximate="tanh") * u
+    for variant in [ops.LINEAR_MFMA] + ([ops.LINEAR_SKINNY] if M <= 64 else []):
+        y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, variant=variant, full_precision=False)
+        close(y, ref, 2e-2, 2 ** -7)
+
+
+def test_linear_mfma_rows_do_not_depend_on_the_batch():
+    # a token's output is the same whatever else is in the batch, within each kernel
+    x, w = rnd(64, 320, seed=20, dtype=torch.bfloat16), rnd(208, 320, seed=21, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    def run(xx, variant):
+        y = torch.empty(xx.shape[0], 208, dtype=torch.float32, device=DEV)
+        ops.linear(xx, wf, y, n_out=208, k_in=320, layout=ops.LAYOUT_FRAG16, variant=variant, full_precision=False)
+        return y
+    for variant in (ops.LINEAR_SKINNY, ops.LINEAR_MFMA):
+        full = run(x, variant)
+        assert torch.equal(run(x[5:6].contiguous(), variant)[0], full[5])
+        assert torch.equal(run(x[:33].contiguous(), variant), full[:33])
+
+
+def test_embed_from_fragment_layout():
+    V, H = 301, 72
+    table = rnd(V, H, seed=1, dtype=torch.bfloat16)
+    tok = torch.tensor([0, 300, 5, 5, 17, 16, 15], dtype=torch.int32, device=DEV)
+    out = torch.empty(7, H, device=DEV)
+    ops.embed(tok, ops.to_frag16(table), out, 3.25, V, H, ops.LAYOUT_FRAG16)
+    close(out, table.double()[tok.long()] * 3.25, 1e-6)
