@@ -55,12 +55,25 @@ int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool
                            const float* cos_t, const float* sin_t, const int* positions,
                            const int* seq_of_token, const int* block_table, int bt_stride, int T,
                            int row_width, int nH, int nKV, int d, int rotary_dim, int page_size, int n_pages,
-                           hipStream_t stream);
+                           int kv_layout, hipStream_t stream);
 
 int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
                             const int* positions, const int* seq_of_token, const int* block_table,
                             int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
                             float softcap, int window, int full_precision, hipStream_t stream);
+
+// bfloat16 attention on the matrix cores over a cache in the fragment layout (kv_layout 1 of
+// alice_rope_cache_write): prompts, and single tokens with the keys split over `splits` blocks.
+int alice_attention_mfma_supported(int d);
+int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
+                            const int* cu_seqlens, const int* context_lens, const int* block_table,
+                            int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
+                            float scale, float softcap, int window, hipStream_t stream);
+long alice_attention_decode_workspace(int B, int nH, int d, int splits);
+int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
+                           const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
+                           int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
+                           hipStream_t stream);
 
 // Lowest index among equal maxima.
 int alice_argmax(const float* logits, int* out, int B, int V, hipStream_t stream);

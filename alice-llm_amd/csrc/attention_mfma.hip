@@ -1,0 +1,335 @@
+// bfloat16 attention over the paged cache on the matrix cores (MFMA 16x16x32, 32-bit softmax),
+// for prompts (flash-style, causal, windowed) and for single decoded tokens (keys split over
+// blocks, parts combined in a fixed order).
+//
+// Order of operations as in the reference (llama3.rs:5622-5688): dot product, times scale, softcap
+// cap * tanh(s / cap), mask to the keys max(0, pos + 1 - window) .. pos (llama3.rs:5444-5451),
+// softmax with a running maximum (llama3.rs:5568-5620), weighted sum of the values; the kv head of
+// query head h is h / (nH / nKV).
+//
+// Cache layout ("fragment" layout, written by rope_cache_write): a page holds 64 positions of one kv
+// head.  Keys:   [key tile t (4)][d tile (d/32)][lane 64][8]: lane g*16 + r holds K[16 t + r][32 dt + 8g ..+8].
+// Values: [key block b (2)][dv tile (d/16)][lane 64][8]: lane g*16 + r, element j holds
+//         V[32 b + 16 (j/4) + 4 g + j%4][16 dvt + r].
+// With keys as the MFMA's first operand and queries as the second, lane l of the score tile holds
+// S[key 4(l/16) + i][query l%16]; two such tiles, rounded to bfloat16, are exactly the second operand
+// of the value product in the key order that the value layout above stores, so the probabilities
+// never move between lanes.  Each lane keeps the running maximum and sum of its query column.
+#include "common.h"
+#include "alice_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)f32_to_bf16(a).bits | ((uint32_t)f32_to_bf16(b).bits << 16);
+}
+// max / sum over the four lanes that hold the same query column (l, l^16, l^32, l^48)
+__device__ __forceinline__ float col_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float col_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+// Running state of NB query tiles (16 query columns each) against the keys seen so far.
+template <int DT, int NB>
+struct Core {
+  u32x4 q[NB][DT];          // query fragments: lane (col, g) holds Q[col][32 dt + 8g ..+8]
+  f32x4 o[NB][2 * DT];      // output^T tiles: lane holds O[dv 16 t + 4(l/16) + i][col l%16]
+  float m[NB], l[NB];       // running maximum and sum of this lane's column
+
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      m[b] = -INFINITY;
+      l[b] = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2 * DT; ++t) o[b][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  // One block of 32 keys: kpage/vpage point at the page of one kv head, kb is the block within the
+  // page (0/1), key0 the absolute position of its first key.  pos[b]: the position of this lane's
+  // query column in tile b (negative: no query).  Keys outside [pos + 1 - window, pos] are masked.
+  __device__ __forceinline__ void block32(const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage, int kb,
+                                          int key0, const int* pos, int window, float scale, float cap, int lane) {
+    const int g = lane >> 4;
+    f32x4 s[NB][2];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(kpage + ((size_t)((kb * 2 + t) * DT + dt) * 64 + lane) * 8);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) s[b][t] = mfma16(kf, q[b][dt], s[b][t]);
+      }
+    u32x4 p[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int lo = window > 0 ? pos[b] + 1 - window : 0;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = key0 + t * 16 + g * 4 + i;
+          float v = s[b][t][i] * scale;
+          if (cap > 0.f) v = cap * tanh_fast(v / cap);
+          v = (key <= pos[b] && key >= lo) ? v : -INFINITY;
+          s[b][t][i] = v;
+          mx = fmaxf(mx, v);
+        }
+      const float m_new = fmaxf(m[b], col_max(mx));
+      const float corr = (m[b] == -INFINITY) ? 0.f : __expf(m[b] - m_new);       // m_new >= m[b]
+      const float base = (m_new == -INFINITY) ? 0.f : m_new;                    // all masked so far: p = exp(-inf) = 0
+      float sum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = __expf(s[b][t][i] - base);
+          s[b][t][i] = e;
+          sum += e;
+        }
+      l[b] = l[b] * corr + col_sum(sum);
+      m[b] = m_new;
+      p[b] = u32x4{pack2(s[b][0][0], s[b][0][1]), pack2(s[b][0][2], s[b][0][3]),
+                   pack2(s[b][1][0], s[b][1][1]), pack2(s[b][1][2], s[b][1][3])};
+      if (corr != 1.f) {
+#pragma unroll
+        for (int t = 0; t < 2 * DT; ++t) o[b][t] *= corr;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t) {
+      const u32x4 vf = *reinterpret_cast<const u32x4*>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) o[b][t] = mfma16(vf, p[b], o[b][t]);
+    }
+  }
+};
+
+// ---------------------------------------------------------------- prompts
+// grid: (tiles of 64 query tokens, sequences, kv heads); 4 waves, wave w takes tokens 16 w .. 16 w + 15
+// of the tile for GH query heads at a time (both share the kv head), looping over the group's heads.
+template <int DT, int GH>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
+  constexpr int D = DT * 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int b = blockIdx.y, kvh = blockIdx.z;
+  const int t_begin = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_begin;
+  const int first = blockIdx.x * 64 + wave * 16;            // this wave's first token within the sequence's new tokens
+  if (first >= n_new) return;
+  const int start_len = context_lens[b] - n_new;
+  const int my_tok = first + col;
+  const bool tok_ok = my_tok < n_new;
+  const int my_pos = tok_ok ? start_len + my_tok : -1;
+  const int last_pos = start_len + min(first + 15, n_new - 1);
+  const int first_key = window > 0 ? max(0, start_len + first + 1 - window) : 0;
+  const int* bt = block_table + (size_t)b * bt_stride;
+  const int group = nH / nKV;
+  const size_t page_elems = (size_t)64 * D;
+
+  for (int h0 = 0; h0 < group; h0 += GH) {
+    Core<DT, GH> c;
+    c.init();
+    int pos[GH];
+#pragma unroll
+    for (int hh = 0; hh < GH; ++hh) {
+      const int head = kvh * group + h0 + hh;
+      const bool ok = tok_ok && (h0 + hh) < group;
+      pos[hh] = ok ? my_pos : -1;
+      const bf16_t* qrow = q + ((size_t)(t_begin + (tok_ok ? my_tok : 0)) * nH + (ok ? head : kvh * group)) * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        c.q[hh][dt] = u32x4{0u, 0u, 0u, 0u};
+        if (ok) c.q[hh][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
+      }
+    }
+    for (int kb32 = first_key >> 5; kb32 <= (last_pos >> 5); ++kb32) {
+      const int page = bt[kb32 >> 1];
+      const bf16_t* kp = k_pool + ((size_t)page * nKV + kvh) * page_elems;
+      const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems;
+      c.block32(kp, vp, kb32 & 1, kb32 << 5, pos, window, scale, cap, lane);
+    }
+#pragma unroll
+    for (int hh = 0; hh < GH; ++hh) {
+      if (pos[hh] < 0) continue;
+      const int head = kvh * group + h0 + hh;
+      const float inv = 1.f / c.l[hh];
+      bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
+#pragma unroll
+      for (int t = 0; t < 2 * DT; ++t) {
+        const f32x4 v = c.o[hh][t] * inv;
+        uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+        *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- single tokens, keys split over blocks
+// grid: (sequences, kv heads, splits).  The query tile's 16 columns are the query heads of the kv head's
+// group (group <= 16).  The sequence's 32-key blocks are dealt out in contiguous runs to the
+// splits * 4 waves; every wave keeps a running (max, sum, output); the block's four waves are combined
+// in LDS in the order 0, 1, 2, 3 and the split's result goes to `parts`:
+// [sequence][head][split][D + 2] = (max, sum, unnormalised output).  With one split the output is final.
+template <int DT>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    bf16_t* __restrict__ out, float* __restrict__ parts, const int* __restrict__ context_lens,
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int splits) {
+  constexpr int D = DT * 32;
+  __shared__ float sm[4][16], sl[4][16];
+  extern __shared__ __align__(16) float so[];            // [4 waves][group][D + 4]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int group = nH / nKV;
+  const int pos = context_lens[b] - 1;
+  const int first_key = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int kb_first = first_key >> 5, kb_last = pos >> 5;
+  const int n_blocks = kb_last - kb_first + 1;
+  const int workers = splits * 4, me = split * 4 + wave;
+  const int per = (n_blocks + workers - 1) / workers;
+  const int my_first = kb_first + me * per, my_last = min(kb_last, my_first + per - 1);
+  const int* bt = block_table + (size_t)b * bt_stride;
+  const size_t page_elems = (size_t)64 * D;
+
+  Core<DT, 1> c;
+  c.init();
+  const bool head_ok = col < group;
+  int cpos[1] = {head_ok ? pos : -1};
+  {
+    const bf16_t* qrow = q + ((size_t)b * nH + kvh * group + (head_ok ? col : 0)) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      c.q[0][dt] = u32x4{0u, 0u, 0u, 0u};
+      if (head_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
+    }
+  }
+  for (int kb32 = my_first; kb32 <= my_last; ++kb32) {
+    const int page = bt[kb32 >> 1];
+    const bf16_t* kp = k_pool + ((size_t)page * nKV + kvh) * page_elems;
+    const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems;
+    c.block32(kp, vp, kb32 & 1, kb32 << 5, cpos, window, scale, cap, lane);
+  }
+  // combine the four waves
+  if (g == 0) { sm[wave][col] = c.m[0]; sl[wave][col] = c.l[0]; }
+  if (head_ok) {
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t)
+      *reinterpret_cast<f32x4*>(&so[((size_t)wave * group + col) * (D + 4) + t * 16 + g * 4]) = c.o[0][t];
+  }
+  __syncthreads();
+  // thread -> (head column hc, dims): 256 threads cover 16 columns x D dims
+  for (int idx = threadIdx.x; idx < 16 * D; idx += 256) {
+    const int hc = idx / D, e = idx % D;
+    if (hc >= group) continue;
+    float mm = fmaxf(fmaxf(sm[0][hc], sm[1][hc]), fmaxf(sm[2][hc], sm[3][hc]));
+    float acc = 0.f, ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = (sm[w][hc] == -INFINITY) ? 0.f : __expf(sm[w][hc] - mm);
+      acc += so[((size_t)w * group + hc) * (D + 4) + e] * f;
+      ll += sl[w][hc] * f;
+    }
+    const int head = kvh * group + hc;
+    if (splits == 1) {
+      out[((size_t)b * nH + head) * D + e] = f32_to_bf16(acc / ll);
+    } else {
+      float* pr = parts + (((size_t)b * nH + head) * splits + split) * (D + 2);
+      pr[2 + e] = acc;
+      if (e == 0) { pr[0] = mm; pr[1] = ll; }
+    }
+  }
+}
+
+// Combines the splits of one (sequence, head) in the order 0, 1, ...: grid (sequences * heads), D threads.
+__global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits) {
+  const float* pr = parts + (size_t)blockIdx.x * splits * (D + 2);
+  float mm = -INFINITY;
+  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[(size_t)s * (D + 2)]);
+  for (int e = threadIdx.x; e < D; e += blockDim.x) {
+    float acc = 0.f, ll = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float* ps = pr + (size_t)s * (D + 2);
+      const float f = (ps[0] == -INFINITY) ? 0.f : __expf(ps[0] - mm);
+      acc += ps[2 + e] * f;
+      ll += ps[1] * f;
+    }
+    out[(size_t)blockIdx.x * D + e] = f32_to_bf16(acc / ll);
+  }
+}
+
+}  // namespace
+
+// Head sizes the matrix-core kernels and the fragment cache layout cover.
+extern "C" int alice_attention_mfma_supported(int d) { return d == 64 || d == 128 || d == 256; }
+
+extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
+                                       const int* cu_seqlens, const int* context_lens, const int* block_table,
+                                       int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
+                                       float scale, float softcap, int window, hipStream_t stream) {
+  ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
+  ALICE_CHECK(nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
+  ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
+  ALICE_CHECK(B >= 0 && max_new >= 0 && B <= 65535 && nKV <= 65535, "attention: bad batch B=%d", B);
+  ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
+  if (B == 0 || max_new == 0) return 0;
+  dim3 grid(ceil_div(max_new, 64), B, nKV);
+  const int group = nH / nKV;
+#define GO(DT, GH) attn_prefill_kernel<DT, GH><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+      (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window)
+  if (d == 64) { if (group % 2 == 0) GO(2, 2); else GO(2, 1); }
+  else if (d == 128) { if (group % 2 == 0) GO(4, 2); else GO(4, 1); }
+  else { if (group % 2 == 0) GO(8, 2); else GO(8, 1); }
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
+// Number of float32 elements `parts` must hold for a decode call.
+extern "C" long alice_attention_decode_workspace(int B, int nH, int d, int splits) {
+  return splits <= 1 ? 0 : (long)B * nH * splits * (d + 2);
+}
+
+extern "C" int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
+                                      const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
+                                      int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
+                                      hipStream_t stream) {
+  ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
+  ALICE_CHECK(nKV >= 1 && nH % nKV == 0 && nH / nKV <= 16, "attention (decode): %d query heads per kv head are more than the 16 this kernel takes", nKV ? nH / nKV : 0);
+  ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
+  ALICE_CHECK(B >= 0 && nKV <= 65535 && splits >= 1 && splits <= 64, "attention: bad batch B=%d or splits=%d", B, splits);
+  ALICE_CHECK(splits == 1 || parts != nullptr, "attention: split keys need the workspace");
+  ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
+  if (B == 0) return 0;
+  dim3 grid(B, nKV, splits);
+  const size_t lds = (size_t)4 * (nH / nKV) * (d + 4) * sizeof(float);
+#define GO(DT) attn_decode_kernel<DT><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+      (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits)
+  if (d == 64) GO(2); else if (d == 128) GO(4); else GO(8);
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  if (splits > 1) {
+    attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits);
+    ALICE_LAUNCH_CHECK();
+  }
+  return 0;
+}

@@ -7,6 +7,20 @@
 #include "common.h"
 #include "alice_hip.h"
 
+// Offsets of element e of the token at place t of a 64-position page of one kv head.  Layout 0 is
+// row-major [position][d]; layout 1 is the fragment layout that the matrix-core attention kernels
+// read (see attention_mfma.hip): keys in 16-position x 32-dim tiles, values in 32-position x 16-dim
+// tiles with the positions in the order the score tiles come out of the MFMA.
+__device__ __forceinline__ size_t k_offset(int layout, int t, int e, int d) {
+  if (layout == 0) return (size_t)t * d + e;
+  return ((size_t)((t >> 4) * (d >> 5) + (e >> 5)) * 64 + ((e & 31) >> 3) * 16 + (t & 15)) * 8 + (e & 7);
+}
+__device__ __forceinline__ size_t v_offset(int layout, int t, int e, int d) {
+  if (layout == 0) return (size_t)t * d + e;
+  const int tt = t & 31, w = tt & 15;
+  return ((size_t)((t >> 5) * (d >> 4) + (e >> 4)) * 64 + (w >> 2) * 16 + (e & 15)) * 8 + ((tt >> 4) * 4 + (w & 3));
+}
+
 // One block per token.  qkv row of row_w elements: [nH*d | nKV*d | nKV*d | ...]; with no pools
 // only the q part is read.  cos/sin: [max_pos, R/2].
 // Cache pools: [page][nKV][page_size][d]; the page of position p of sequence s is
@@ -17,7 +31,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                   const int* __restrict__ block_table, int bt_stride, int row_w,
-                                  int nH, int nKV, int d, int R, int page_size, int n_pages) {
+                                  int nH, int nKV, int d, int R, int page_size, int n_pages, int layout) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = R >> 1;
@@ -25,13 +39,14 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
   const float* cs = cos_t ? cos_t + (size_t)pos * half : nullptr;
   const float* sn = sin_t ? sin_t + (size_t)pos * half : nullptr;
 
-  T* kdst = nullptr;
+  T* kdst = nullptr;             // the page's region of kv head 0; head h adds h * page_size * d
   T* vdst = nullptr;
+  const int tp = pos % page_size;  // place within the page
   if (k_pool) {
     const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
     if (page >= 0 && page < n_pages) {
-      const size_t base = ((size_t)page * nKV * page_size + (size_t)(pos % page_size)) * d;
-      kdst = k_pool + base;      // head h adds h * page_size * d
+      const size_t base = (size_t)page * nKV * page_size * d;
+      kdst = k_pool + base;
       vdst = v_pool + base;
     }
   }
@@ -49,23 +64,25 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
       if (!kdst) continue;
       dst = kdst + (size_t)(h - nH) * page_size * d;
     }
+    // where element e goes: q rows are plain; k goes to its place in the page
+    auto at = [&](int e) -> size_t { return is_q ? (size_t)e : k_offset(layout, tp, e, d); };
     // Elements of this item: the rotated pair (j, j + half) if j < half, and the pass-through
     // elements are handled by the items with j >= half: each copies e = half + j and, when
     // R < d, nothing is lost because e ranges over [2*half .. ) below.
     if (j < half) {
       float x0 = load_f32(src, j), x1 = load_f32(src, j + half);
       float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
-      store_f32(dst, j, x0 * c - x1 * s);
-      store_f32(dst, j + half, x0 * s + x1 * c);
+      store_f32(dst, at(j), x0 * c - x1 * s);
+      store_f32(dst, at(j + half), x0 * s + x1 * c);
     }
     // pass-through elements: indices R .. d-1, spread over the items j of this head
-    for (int e = R + j; e < d; e += hd2) store_f32(dst, e, load_f32(src, e));
+    for (int e = R + j; e < d; e += hd2) store_f32(dst, at(e), load_f32(src, e));
   }
   if (vdst) {
     const T* vsrc = row + (size_t)(nH + nKV) * d;
     for (int it = threadIdx.x; it < nKV * d; it += blockDim.x) {
       const int h = it / d, e = it % d;
-      vdst[(size_t)h * page_size * d + e] = vsrc[it];
+      vdst[(size_t)h * page_size * d + v_offset(layout, tp, e, d)] = vsrc[it];
     }
   }
 }
@@ -74,7 +91,7 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
                                       const float* cos_t, const float* sin_t, const int* positions,
                                       const int* seq_of_token, const int* block_table, int bt_stride,
                                       int T, int row_width, int nH, int nKV, int d, int rotary_dim, int page_size,
-                                      int n_pages, hipStream_t stream) {
+                                      int n_pages, int kv_layout, hipStream_t stream) {
   ALICE_CHECK(dtype_ok(dtype), "rope: unknown dtype %d", dtype);
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 2 && d % 2 == 0, "rope: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
   ALICE_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0, "rope: rotated width %d must be even and at most head_dim %d", rotary_dim, d);
@@ -84,10 +101,12 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
   ALICE_CHECK(k_pool == nullptr || (block_table && seq_of_token && page_size > 0 && n_pages > 0 && nKV >= 1),
               "rope: a cache write needs the block table, the token-to-sequence map and the page geometry");
   ALICE_CHECK(row_width >= (nH + (k_pool ? 2 * nKV : 0)) * d, "rope: rows of %d elements are too short for the heads", row_width);
+  ALICE_CHECK(kv_layout == 0 || (kv_layout == 1 && page_size == 64 && d % 32 == 0 && dtype == DT_BF16) || k_pool == nullptr,
+              "rope: the fragment cache layout needs bfloat16, pages of 64 and head_dim %% 32 == 0");
   if (T == 0) return 0;
   DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<T, 256, 0, stream>>>(
       (const TT*)qkv, (TT*)q_out, (TT*)k_pool, (TT*)v_pool, cos_t, sin_t, positions, seq_of_token,
-      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages)));
+      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout)));
   ALICE_LAUNCH_CHECK();
   return 0;
 }

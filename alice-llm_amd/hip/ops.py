@@ -42,7 +42,10 @@ def _declare(lib) -> None:
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
         "alice_frag16_supported": [I, I, I],
-        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
+        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P],
+        "alice_attention_mfma_supported": [I],
+        "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
+        "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, I, I, P],
         "alice_sample": [P, P, P, I, I, F, I, F, P],
@@ -77,6 +80,12 @@ def library():
                                   f"need {ABI_VERSION}: rebuild it (python -m alice_llm_amd.csrc.build)")
         _lib = lib
         return _lib
+
+
+def library_ready() -> bool:
+    """Whether kernels can run at all here (a GPU is visible); skeleton models built on the CPU to list
+    their tensors do not touch the library."""
+    return torch.cuda.is_available()
 
 
 def library_path() -> Optional[str]:
@@ -231,7 +240,7 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
                      v_pool: Optional[torch.Tensor], cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                      positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
                      block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
-                     rotary_dim: int, max_position: int) -> None:
+                     rotary_dim: int, max_position: int, kv_layout: int = 0) -> None:
     """Rotate q and k; write k and v at their positions into the pools [pages, nKV, page, d].
     With k_pool None the row holds q only (num_kv_heads = 0) and nothing is cached.
     `max_position` is the largest position among `positions` (the host knows it): checked against the tables."""
@@ -267,7 +276,7 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
     _call("alice_rope_cache_write", qkv.data_ptr(), dtype_code(dt), q_out.data_ptr(), _opt(k_pool, "k_pool"),
           _opt(v_pool, "v_pool"), _opt(cos, "cos"), _opt(sin, "sin"), positions.data_ptr(),
           _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T, row_width, num_heads,
-          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, _stream())
+          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, int(kv_layout), _stream())
 
 
 def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor,
@@ -299,11 +308,77 @@ def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
     return bool(library().alice_frag16_supported(int(rows), int(k_in), int(epilogue)))
 
 
+KV_ROW, KV_FRAGMENT = 0, 1
+
+
+def attention_mfma_supported(head_dim: int) -> bool:
+    """Whether the matrix-core attention kernels (and the fragment cache layout) cover this head size."""
+    return bool(library().alice_attention_mfma_supported(int(head_dim)))
+
+
+def decode_splits(n_seqs: int, num_kv_heads: int, max_context: int) -> int:
+    """Into how many blocks the keys of a sequence are split for single-token attention: enough to
+    fill the chip (about a thousand waves), at least eight 32-key blocks per block of four waves."""
+    by_fill = -(-1024 // max(1, n_seqs * num_kv_heads * 4))
+    by_work = max(1, -(-max_context // 32) // 8)
+    return max(1, min(by_fill, by_work, 64))
+
+
+def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_table, *, num_heads: int, n_seqs: int,
+                      max_new: int, max_context: int, scale: float, softcap: Optional[float], window: Optional[int]) -> None:
+    n_pages, nKV, page_size, d = k_pool.shape
+    T = q.shape[0]
+    _dev(q, "q", torch.bfloat16, (T, num_heads * d))
+    _dev(out, "out", torch.bfloat16, (T, num_heads * d))
+    _dev(k_pool, "k_pool", torch.bfloat16)
+    _dev(v_pool, "v_pool", torch.bfloat16, k_pool.shape)
+    _dev(cu_seqlens, "cu_seqlens", torch.int32, (n_seqs + 1,))
+    _dev(context_lens, "context_lens", torch.int32, (n_seqs,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or block_table.shape[0] < n_seqs or (max_context - 1) // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"{max_context} keys are beyond the block table {tuple(block_table.shape)}")
+    _call("alice_attention_prefill", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
+          cu_seqlens.data_ptr(), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_seqs,
+          max_new, num_heads, nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), _stream())
+
+
+def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,
+                     scale: float, softcap: Optional[float], window: Optional[int], splits: Optional[int] = None) -> None:
+    n_pages, nKV, page_size, d = k_pool.shape
+    B = q.shape[0]
+    _dev(q, "q", torch.bfloat16, (B, num_heads * d))
+    _dev(out, "out", torch.bfloat16, (B, num_heads * d))
+    _dev(k_pool, "k_pool", torch.bfloat16)
+    _dev(v_pool, "v_pool", torch.bfloat16, k_pool.shape)
+    _dev(context_lens, "context_lens", torch.int32, (B,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or block_table.shape[0] < B or (max_context - 1) // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"{max_context} keys are beyond the block table {tuple(block_table.shape)}")
+    if splits is None:
+        reach = max_context if not window else min(max_context, window + 32)
+        splits = decode_splits(B, nKV, reach)
+    parts = torch.empty((B * num_heads * splits * (d + 2),), dtype=torch.float32, device=q.device) if splits > 1 else None
+    _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
+          _opt(parts, "parts"), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], B, num_heads,
+          nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, _stream())
+
+
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,
               block_table: torch.Tensor, *, num_heads: int, scale: float, softcap: Optional[float],
-              window: Optional[int], full_precision: bool) -> None:
-    """Attention of the step's query tokens over the cache; picks the kernel for the step's shape.
-    `ctx` carries positions, seq_of_token, max_position (and the prompt/decode shape of the step)."""
+              window: Optional[int], full_precision: bool, kv_layout: int = KV_ROW) -> None:
+    """Attention of the step's query tokens over the cache; picks the kernel for the step's shape and
+    the cache's layout.  `ctx` carries positions, seq_of_token, cu_seqlens, context_lens and the
+    host-side sizes of the step."""
+    if kv_layout == KV_FRAGMENT:
+        nKV = k_pool.shape[1]
+        if ctx.is_decode and num_heads // nKV <= 16:
+            attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
+                             max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
+        else:
+            attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
+                              num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
+                              max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
+        return
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
                       max_position=ctx.max_position, full_precision=full_precision)

@@ -36,6 +36,11 @@ class Attention(Part):
         self.q_dim, self.kv_dim = num_heads * head_dim, num_kv_heads * head_dim
         self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, precision)
         self.o = Linear(self.q_dim, hidden_size, precision)
+        # How this mixer lays keys and values out inside a page: the matrix-core kernels read a fragment
+        # layout; every other case is row-major.  It depends on the arithmetic and the head size alone, so
+        # that a run that reads another run's cache finds the layout it expects.
+        self.kv_layout = (ops.KV_FRAGMENT if precision.name == "bfloat16" and precision.act == torch.bfloat16
+                          and ops.library_ready() and ops.attention_mfma_supported(head_dim) else ops.KV_ROW)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -70,8 +75,9 @@ class Attention(Part):
         qkv = self.qkv(x, self.precision.act)
         q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
         self.position.rotate_and_store(qkv, q, ctx, cache, num_heads=self.nH, num_kv_heads=self.nKV,
-                                       head_dim=self.d)
+                                       head_dim=self.d, kv_layout=self.kv_layout)
         out = torch.empty_like(q)
         ops.attention(q, cache.k, cache.v, out, ctx, cache.block_table, num_heads=self.nH, scale=self.scale,
-                      softcap=self.softcap, window=self.window, full_precision=self.precision.full)
+                      softcap=self.softcap, window=self.window, full_precision=self.precision.full,
+                      kv_layout=self.kv_layout)
         return self.o(out, torch.float32, allow_partials=True)

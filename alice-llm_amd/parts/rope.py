@@ -34,13 +34,13 @@ class RotaryEncoding(Part):
         self.sin = torch.sin(ang).to(torch.float32).to(device).contiguous()
 
     def rotate_and_store(self, qkv: torch.Tensor, q_out: torch.Tensor, ctx, cache, *, num_heads: int,
-                         num_kv_heads: int, head_dim: int) -> None:
+                         num_kv_heads: int, head_dim: int, kv_layout: int = 0) -> None:
         write = cache is not None and cache.writable
         ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None,
                              self.cos, self.sin, ctx.positions, ctx.seq_of_token if write else None,
                              cache.block_table if write else None, num_heads=num_heads,
                              num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=self.rotary_dim,
-                             max_position=ctx.max_position)
+                             max_position=ctx.max_position, kv_layout=kv_layout)
 
 
 @POSITIONS.register("none")
@@ -50,10 +50,10 @@ class NoPositionEncoding(Part):
     def __init__(self, precision: Precision, device, **_):
         pass
 
-    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim) -> None:
+    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim, kv_layout=0) -> None:
         write = cache is not None and cache.writable
         ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None, None, None,
                              ctx.positions, ctx.seq_of_token if write else None,
                              cache.block_table if write else None, num_heads=num_heads,
                              num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=0,
-                             max_position=ctx.max_position)
+                             max_position=ctx.max_position, kv_layout=kv_layout)

@@ -388,3 +388,122 @@ def test_embed_from_fragment_layout():
     out = torch.empty(7, H, device=DEV)
     ops.embed(tok, ops.to_frag16(table), out, 3.25, V, H, ops.LAYOUT_FRAG16)
     close(out, table.double()[tok.long()] * 3.25, 1e-6)
+
+
+# ------------------------------------------------------------------ matrix-core attention over the fragment cache layout
+def frag_case(nH, nKV, d, lens, new, cap, window, seed, crafted=None):
+    """Like attention_case, with the cache filled by rope_cache_write in the fragment layout (no rotation)."""
+    B = len(lens)
+    kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, B, seed)
+    qs, refs = [], []
+    scale = 1.0 / math.sqrt(d * 1.7)
+    for b, (L, n) in enumerate(zip(lens, new)):
+        g = torch.Generator().manual_seed(seed * 100 + b)
+        q = torch.randn(L, nH, d, generator=g, dtype=D)
+        k = torch.randn(L, nKV, d, generator=g, dtype=D)
+        v = torch.randn(L, nKV, d, generator=g, dtype=D)
+        if crafted is not None:
+            crafted(b, q, k, v)
+        q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
+        qkv = torch.cat([q.reshape(L, -1), k.reshape(L, -1), v.reshape(L, -1)], dim=1).contiguous().to(DEV)
+        pos = torch.arange(L, dtype=torch.int32, device=DEV)
+        ops.rope_cache_write(qkv, torch.empty(L, nH * d, dtype=torch.bfloat16, device=DEV), kp, vp, None, None, pos,
+                             torch.full((L,), b, dtype=torch.int32, device=DEV), bt, num_heads=nH, num_kv_heads=nKV,
+                             head_dim=d, rotary_dim=0, max_position=L - 1, kv_layout=ops.KV_FRAGMENT)
+        refs.append(P.attention_core(q.double(), k.double(), v.double(), scale, cap, window)[L - n:])
+        qs.append(q[L - n:])
+    q = torch.cat(qs).reshape(-1, nH * d).to(DEV)
+    cu = [0]
+    for n in new:
+        cu.append(cu[-1] + n)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    return q, kp, vp, bt, i32(cu), i32(list(lens)), torch.cat(refs).reshape(-1, nH * d), scale
+
+
+FRAG_SHAPES = [(6, 2, 64), (4, 4, 64), (8, 4, 256), (4, 1, 128), (3, 3, 128), (32, 16, 128)]
+
+
+def test_fragment_cache_layout_is_what_the_comment_says():
+    nKV, d, L = 2, 64, 70
+    kp, vp, bt = paged(L, nKV, d, torch.bfloat16, 1, seed=30)
+    k = rnd(L, nKV, d, seed=31, dtype=torch.bfloat16)
+    v = rnd(L, nKV, d, seed=32, dtype=torch.bfloat16)
+    qkv = torch.cat([torch.zeros(L, d, dtype=torch.bfloat16, device=DEV), k.reshape(L, -1), v.reshape(L, -1)], 1).contiguous()
+    ops.rope_cache_write(qkv, torch.empty(L, d, dtype=torch.bfloat16, device=DEV), kp, vp, None, None,
+                         torch.arange(L, dtype=torch.int32, device=DEV), torch.zeros(L, dtype=torch.int32, device=DEV), bt,
+                         num_heads=1, num_kv_heads=nKV, head_dim=d, rotary_dim=0, max_position=L - 1, kv_layout=ops.KV_FRAGMENT)
+    for t, h, e in ((0, 0, 0), (17, 1, 37), (63, 0, 63), (64, 1, 5), (69, 0, 48), (33, 1, 16)):
+        page, tp = int(bt[0, t // 64]), t % 64
+        kflat, vflat = kp[page, h].reshape(-1), vp[page, h].reshape(-1)
+        koff = (((tp // 16) * (d // 32) + e // 32) * 64 + ((e % 32) // 8) * 16 + tp % 16) * 8 + e % 8
+        w = tp % 16
+        voff = (((tp // 32) * (d // 16) + e // 16) * 64 + (w // 4) * 16 + e % 16) * 8 + (((tp % 32) // 16) * 4 + w % 4)
+        assert kflat[koff] == k[t, h, e] and vflat[voff] == v[t, h, e]
+
+
+@pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
+@pytest.mark.parametrize("cap,window", [(None, None), (5.0, 50), (50.0, 7), (2.0, 64)])
+def test_attention_mfma_prompts(nH, nKV, d, cap, window):
+    for lens, new in (((5, 130, 66), (5, 130, 66)), ((150, 64, 33), (20, 3, 33)), ((300,), (300,))):
+        q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, new, cap, window, seed=3)
+        out = torch.full_like(q, float("nan"))
+        ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
+                              max_context=max(lens), scale=scale, softcap=cap, window=window)
+        close(out, ref, 2e-2)
+
+
+@pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
+@pytest.mark.parametrize("cap,window", [(None, None), (5.0, 50), (50.0, 7), (2.0, 64)])
+def test_attention_mfma_single_tokens(nH, nKV, d, cap, window):
+    lens = (200, 1, 77, 64, 65, 33, 700)
+    q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, (1,) * len(lens), cap, window, seed=4)
+    for splits in (None, 1, 2, 5, 16):
+        out = torch.full_like(q, float("nan"))
+        ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=cap,
+                             window=window, splits=splits)
+        close(out, ref, 2e-2)
+    # the prompt kernel on single tokens gives the same
+    out = torch.full_like(q, float("nan"))
+    ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=1, max_context=max(lens),
+                          scale=scale, softcap=cap, window=window)
+    close(out, ref, 2e-2)
+
+
+def test_attention_mfma_far_key_and_window_edge():
+    nH, nKV, d, L = 4, 2, 64, 700
+    def far(b, q, k, v):
+        k[3] = 0; k[3, :, 0] = 40.0
+        q[L - 1] = 0; q[L - 1, :, 0] = 40.0
+    q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, None, seed=5, crafted=far)
+    for fn in ("decode", "prefill"):
+        out = torch.full_like(q, float("nan"))
+        if fn == "decode":
+            ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=None)
+        else:
+            ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=1, max_new=1, max_context=L, scale=scale,
+                                  softcap=None, window=None)
+        close(out, ref, 2e-2)
+        assert (out.view(nH, d)[0].double().cpu() - ref.view(nH, d)[0]).abs().max() < 2e-2 and ref.view(nH, d)[0].abs().max() > 0.1
+    for where, seen in ((L - 101, False), (L - 100, True)):
+        def edge(b, q, k, v, where=where):
+            k[where] = 0; k[where, :, 0] = 40.0; v[where] = 7.0
+            q[L - 1] = 0; q[L - 1, :, 0] = 40.0
+        q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, 100, seed=6, crafted=edge)
+        for fn in ("decode", "prefill"):
+            out = torch.full_like(q, float("nan"))
+            if fn == "decode":
+                ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=100)
+            else:
+                ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=1, max_new=1, max_context=L,
+                                      scale=scale, softcap=None, window=100)
+            close(out, ref, 2e-2)
+            assert (abs(float(out[0, 0]) - 7.0) < 5e-2) == seen
+
+
+def test_attention_mfma_refuses_other_head_sizes():
+    assert ops.attention_mfma_supported(256) and not ops.attention_mfma_supported(24) and not ops.attention_mfma_supported(96)
+    kp = torch.zeros(2, 1, 64, 96, dtype=torch.bfloat16, device=DEV)
+    q = torch.zeros(1, 96, dtype=torch.bfloat16, device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    with pytest.raises(ops.HipLibraryError, match="head_dim 96 is not covered"):
+        ops.attention_decode(q, kp, kp, q.clone(), i32([5]), i32([[1]]), num_heads=1, max_context=5, scale=1.0, softcap=None, window=None)
