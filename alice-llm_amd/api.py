@@ -54,8 +54,10 @@ class Model:
         return cls(config, lm)
 
     # ------------------------------------------------------------------ use
-    def engine(self, max_tokens: int, max_seqs: Optional[int] = None) -> Engine:
-        return Engine(self.lm, max_tokens=max_tokens, max_seqs=max_seqs)
+    def engine(self, max_tokens: int, max_seqs: Optional[int] = None, use_graphs: Optional[bool] = None) -> Engine:
+        """A cache sized for max_tokens and the step function over it.  use_graphs: record decode steps into
+        HIP graphs (default: whenever every part of the model allows it)."""
+        return Engine(self.lm, max_tokens=max_tokens, max_seqs=max_seqs, use_graphs=use_graphs)
 
     new_cache = engine
 

@@ -102,16 +102,19 @@ class PageGroup:
             tab.append(self._free.pop())
 
     def trim(self, slot: int, length: int) -> None:
-        """Give back the pages that no query at position >= length can reach."""
+        """Give back the pages that no query at position >= length can reach; True if any was."""
         w = self.need.window
         if w is None:
-            return
+            return False
         first_needed = max(0, length + 1 - w)        # oldest key of the next query
         tab = self._table[slot]
+        changed = False
         for i in range(min(first_needed // self.page_size, len(tab))):
             if tab[i] >= 0:
                 self._free.append(tab[i])
                 tab[i] = -1
+                changed = True
+        return changed
 
     def close(self, slot: int) -> None:
         if slot not in self._table:
@@ -149,6 +152,7 @@ class Cache:
         self.max_tokens = n_pages * page_size
         n_slots = max_seqs if max_seqs is not None else min(n_pages, 4096)
         self.slots = SlotTable(n_slots)
+        self.version = 0                       # bumped whenever any page table changes
         by_need: Dict[KVNeed, List[int]] = {}
         for i, need in enumerate(needs):
             if need is not None and need.kv is not None:
@@ -175,6 +179,7 @@ class Cache:
 
     def close(self, slot: int) -> None:
         self.slots.give_back(slot)
+        self.version += 1
         for g in self.groups:
             g.close(slot)
 
@@ -198,13 +203,16 @@ class Cache:
                     f"layers {g.layers}, {g.n_free()} are free (cache sized for {self.max_tokens} tokens)")
         for g in self.groups:
             for s, l in zip(slots, new_lens):
+                if g.pages_needed(s, l):
+                    self.version += 1
                 g.grow(s, l)
 
     def commit(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
         for s, n in zip(slots, n_new):
             self.slots.advance(s, n)
             for g in self.groups:
-                g.trim(s, self.slots.length(s))
+                if g.trim(s, self.slots.length(s)):
+                    self.version += 1
 
     def block_table_rows(self, group: int, slots: Sequence[int], width: int) -> List[List[int]]:
         g = self.groups[group]

@@ -102,6 +102,14 @@ class CausalLM:
                 total += part.weight.numel() * part.weight.element_size()
         return total
 
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model can be recorded into a HIP graph: every part that runs in a
+        step declares `graph_safe = True` (its launches depend on device data and on sizes fixed per graph)."""
+        parts = [self.embedding, self.head, self.final_norm] + list(self.positions.values())
+        for layer in self.layers:
+            parts += [layer.mixer, layer.feed_forward, layer.block] + list(layer.norms.values())
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+
     # ------------------------------------------------------------------ cache needs
     def _need(self, layer: int):
         mixer = self.layers[layer].mixer

@@ -45,10 +45,86 @@ class StepContext:
 Want = Union[str, Sequence[Sequence[int]]]
 
 
+def _bucket(n: int) -> int:
+    """Batch sizes that share a captured decode step: powers of two up to 64, then multiples of 64."""
+    if n <= 64:
+        b = 1
+        while b < n:
+            b *= 2
+        return b
+    return -(-n // 64) * 64
+
+
+CONTEXT_BUCKET = 512        # captured decode steps are specialised to the context length rounded up to this
+
+
+class _DecodeGraph:
+    """One captured decode step: its static integer inputs, its static logits, and pinned staging buffers."""
+
+    def __init__(self, engine: "Engine", batch: int, context: int):
+        self.batch, self.context = batch, context
+        dev = engine.device
+        self.width = -(-engine.max_positions // engine.cache.page_size)
+        n_groups = len(engine.cache.groups)
+        B = batch
+        sizes = [B, B, B, B, B, B + 1, B] + [B * self.width] * n_groups
+        self.offs = [0]
+        for n in sizes:
+            self.offs.append(self.offs[-1] + n)
+        self.static = torch.zeros(self.offs[-1], dtype=torch.int32, device=dev)
+        self.staging = [torch.zeros(self.offs[-1], dtype=torch.int32).pin_memory() for _ in range(4)]
+        self.events = [None] * 4
+        self.turn = 0
+        part = lambda i: self.static[self.offs[i]:self.offs[i + 1]]
+        self.block_tables = [part(7 + g).view(B, self.width) for g in range(n_groups)]
+        self.ctx = StepContext(tokens=part(0), positions=part(1), seq_of_token=part(2), slots=part(3), want_rows=part(4),
+                               cu_seqlens=part(5), context_lens=part(6), n_tokens=B, n_seqs=B, is_decode=True,
+                               max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
+                               start_lens=[0] * B, slot_ids=[0] * B)
+        self.graph = None
+        self.logits = None
+        self.tables_version = None
+        self.tables_slots = None
+
+    def fill(self, engine: "Engine", slots, tokens, start) -> None:
+        """Write this step's integers into a pinned buffer and queue its copy to the device."""
+        B, n = self.batch, len(slots)
+        i = self.turn = (self.turn + 1) % len(self.staging)
+        if self.events[i] is not None:
+            self.events[i].synchronize()                     # the copy that last used this buffer has run
+        hp = self.staging[i]
+        o = self.offs
+        prev = self.staging[(i - 1) % len(self.staging)]
+        same_tables = (self.tables_version == engine.cache.version and self.tables_slots == list(slots))
+        if same_tables:
+            hp[o[7]:].copy_(prev[o[7]:])
+        else:
+            for g in range(len(self.block_tables)):
+                rows = engine.cache.block_table_rows(g, slots, self.width)
+                flat = [p for r in rows for p in r] + [0] * ((B - n) * self.width)
+                hp[o[7 + g]:o[8 + g]] = torch.tensor(flat, dtype=torch.int32)
+            self.tables_version, self.tables_slots = engine.cache.version, list(slots)
+        pad = B - n
+        hp[o[0]:o[1]] = torch.tensor(list(tokens) + [0] * pad, dtype=torch.int32)
+        hp[o[1]:o[2]] = torch.tensor(list(start) + [0] * pad, dtype=torch.int32)
+        hp[o[6]:o[7]] = torch.tensor([l + 1 for l in start] + [1] * pad, dtype=torch.int32)
+        if self.graph is None:                               # constant parts, written once per buffer set
+            for buf in self.staging:
+                buf[o[2]:o[3]] = torch.arange(B, dtype=torch.int32)
+                buf[o[3]:o[4]] = 0
+                buf[o[4]:o[5]] = torch.arange(B, dtype=torch.int32)
+                buf[o[5]:o[6]] = torch.arange(B + 1, dtype=torch.int32)
+        self.static.copy_(hp, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+
+
 class Engine:
     """A model, its cache, and the step function over them."""
 
-    def __init__(self, model: CausalLM, *, max_tokens: int, max_seqs: Optional[int] = None):
+    def __init__(self, model: CausalLM, *, max_tokens: int, max_seqs: Optional[int] = None,
+                 use_graphs: Optional[bool] = None, max_graphs: int = 24):
         self.model = model
         self.device = model.device
         ops.require_gpu()
@@ -56,6 +132,12 @@ class Engine:
                            device=self.device, max_seqs=max_seqs)
         self.vocab_size = model.plan.vocab_size
         self.max_positions = model.plan.max_positions
+        # Decode steps are captured into HIP graphs when every part says its launches can be recorded
+        # (parts that loop on the host over sequences cannot) and no layer keeps fixed-size state.
+        safe = model.graph_safe() and not self.cache.state
+        self.use_graphs = safe if use_graphs is None else (use_graphs and safe)
+        self._graphs = {}
+        self._max_graphs = max_graphs
 
     # ------------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> List[int]:
@@ -102,6 +184,11 @@ class Engine:
                 raise ValueError("want must give, per sequence, indices into its new tokens")
         self.cache.reserve(slots, n_new)                       # raises before any launch
 
+        if self.use_graphs and want == "last" and max(n_new) == 1:
+            logits = self._graph_step(slots, flat, start)
+            self.cache.commit(slots, n_new)
+            return logits
+
         cu = [0]
         for n in n_new:
             cu.append(cu[-1] + n)
@@ -129,3 +216,31 @@ class Engine:
         logits = self.model.forward(ctx, self.cache, block_tables)
         self.cache.commit(slots, n_new)
         return logits
+
+    # ------------------------------------------------------------------ captured decode steps
+    def _graph_step(self, slots, tokens, start) -> torch.Tensor:
+        """One token per sequence through a captured HIP graph.  The batch is padded to a bucket size with
+        rows that read and write only the cache's spare page; their logits are dropped."""
+        B = len(slots)
+        context = min(self.max_positions, -(-(max(start) + 1) // CONTEXT_BUCKET) * CONTEXT_BUCKET)
+        key = (_bucket(B), context)
+        g = self._graphs.get(key)
+        if g is None:
+            if len(self._graphs) >= self._max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            g = self._graphs[key] = _DecodeGraph(self, key[0], context)
+        else:
+            self._graphs[key] = self._graphs.pop(key)          # most recently used last
+        g.fill(self, slots, tokens, start)
+        if g.graph is None:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.model.forward(g.ctx, self.cache, g.block_tables)      # runs this very step once, eagerly
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                g.logits = self.model.forward(g.ctx, self.cache, g.block_tables)
+            g.graph = graph
+        g.graph.replay()
+        return g.logits[:B].clone()                          # the graph's own buffer is overwritten by its next replay

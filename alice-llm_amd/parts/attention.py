@@ -20,6 +20,8 @@ from .linear import Linear
 
 @MIXERS.register("attention")
 class Attention(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, positions: dict, *, hidden_size: int, num_heads: int,
                  num_kv_heads: int, head_dim: int, scale: float, softcap: Optional[float] = None,
                  window: Optional[int] = None, position: Optional[str] = None):

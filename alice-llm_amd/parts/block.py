@@ -13,6 +13,8 @@ from .base import BLOCKS
 
 @BLOCKS.register("sandwich")
 class SandwichBlock:
+    graph_safe = True
+
     def __init__(self, mixer, feed_forward, norms: Dict[str, object]):
         self.mixer = mixer
         self.feed_forward = feed_forward

@@ -18,6 +18,8 @@ from .linear import Linear
 
 @EMBEDDINGS.register("embedding")
 class Embedding(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, *, vocab_size: int, dim: int, scale: float = 1.0):
         self.precision = precision
         self.V, self.dim, self.scale = vocab_size, dim, float(scale)
@@ -42,6 +44,8 @@ class Embedding(Part):
 
 @HEADS.register("lm_head")
 class OutputHead(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, *, vocab_size: int, dim: int, softcap: Optional[float] = None,
                  tied_to: Optional[str] = None):
         self.precision = precision

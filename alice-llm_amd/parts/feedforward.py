@@ -18,6 +18,8 @@ _GATED_EPILOGUES = {"gelu_tanh": ops.EPI_GEGLU}
 
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, *, hidden_size: int, intermediate_size: int, activation: str):
         if activation not in _GATED_EPILOGUES:
             raise ValueError(f"gated_mlp has no kernel for activation '{activation}'; "

@@ -16,6 +16,8 @@ from .base import NORMS, ParamSpec, Part, Precision
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, *, dim: int, eps: float, weight_offset: float = 0.0):
         self.precision = precision
         self.dim = dim

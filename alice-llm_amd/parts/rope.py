@@ -18,6 +18,8 @@ from .base import POSITIONS, Part, Precision
 
 @POSITIONS.register("rope")
 class RotaryEncoding(Part):
+    graph_safe = True
+
     def __init__(self, precision: Precision, device, *, dim: int, theta: float, max_positions: int,
                  rotary_dim: Optional[int] = None):
         self.dim = dim
@@ -45,6 +47,8 @@ class RotaryEncoding(Part):
 
 @POSITIONS.register("none")
 class NoPositionEncoding(Part):
+    graph_safe = True
+
     """No rotation: q passes through, k and v go to the cache unchanged."""
 
     def __init__(self, precision: Precision, device, **_):

@@ -163,3 +163,42 @@ def test_step_argument_errors():
     with pytest.raises(alice.CacheError, match="all 2 slots"):
         eng.open(1)
     eng.close(s)
+
+
+@pytest.mark.parametrize("name,dtype", [("tiny-c", "bfloat16"), ("tiny-b", "float32")])
+def test_captured_decode_steps_match_eager_on_every_replay(name, dtype):
+    """Decode steps recorded into HIP graphs: every replay is compared with the same step run eagerly, with
+    eager work (a prompt step of another batch, a shrinking batch, a new context bucket) between replays."""
+    model, plain = setup(name, dtype)
+    eager = model.engine(max_tokens=64 * 40, max_seqs=8, use_graphs=False)
+    graph = model.engine(max_tokens=64 * 40, max_seqs=8, use_graphs=True)
+    assert graph.use_graphs and not eager.use_graphs
+    seqs = [random_tokens(plain.V, n, 50 + i) for i, n in enumerate((30, 75, 9, 520, 130))]
+    lens = [10, 60, 3, 500, 100]
+    se, sg = eager.open(5), graph.open(5)
+    for eng, sl in ((eager, se), (graph, sg)):
+        eng.step(sl, [s[:n] for s, n in zip(seqs, lens)], "none")
+    live = list(range(5))
+    step = 0
+    while live:
+        feed = [[seqs[i][lens[i] + step]] for i in live]
+        a = eager.step([se[i] for i in live], feed, "last")
+        b = graph.step([sg[i] for i in live], feed, "last").clone()
+        assert a.shape == b.shape
+        assert max_err(a, b) < (1e-5 if dtype == "float32" else 2e-2), (step, max_err(a, b))
+        if step % 5 == 2:                                    # eager work between replays, on other slots
+            extra = graph.open(1)
+            graph.step(extra, [random_tokens(plain.V, 70, step)], "last")
+            graph.close(extra)
+        step += 1
+        done = [i for i in live if lens[i] + step >= len(seqs[i])]
+        for eng, sl in ((eager, se), (graph, sg)):
+            eng.close([sl[i] for i in done])
+        live = [i for i in live if i not in done]
+    assert len(graph._graphs) >= 3            # batches of 5 (bucket 8), then fewer; a second context bucket past 512
+    ref = plain.forward(seqs[3])
+    s = graph.open(1)
+    graph.step(s, [seqs[3][:500]], "none")
+    got = torch.cat([graph.step(s, [[t]], "last").clone() for t in seqs[3][500:]])
+    assert max_err(got, ref[500:]) < tol(dtype, ref)
+    graph.cache.check_consistent()
