@@ -76,7 +76,8 @@ int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool
                            hipStream_t stream);
 
 // Lowest index among equal maxima.
-int alice_argmax(const float* logits, int* out, int B, int V, hipStream_t stream);
+int alice_argmax_chunks(int B, int V);
+int alice_argmax(const float* logits, int* out, float* work_v, int* work_i, int B, int V, hipStream_t stream);
 // temperature -> top-k (0: off) -> top-p (>= 1: off) -> softmax -> first index whose cumulative
 // probability exceeds uniform[row].
 int alice_sample(const float* logits, int* out, const float* uniform, int B, int V, float temperature,

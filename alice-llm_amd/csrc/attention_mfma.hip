@@ -57,11 +57,26 @@ struct Core {
     }
   }
 
-  // One block of 32 keys: kpage/vpage point at the page of one kv head, kb is the block within the
-  // page (0/1), key0 the absolute position of its first key.  pos[b]: the position of this lane's
-  // query column in tile b (negative: no query).  Keys outside [pos + 1 - window, pos] are masked.
-  __device__ __forceinline__ void block32(const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage, int kb,
-                                          int key0, const int* pos, int window, float scale, float cap, int lane) {
+  // The fragments of one block of 32 keys: kpage/vpage point at the page of one kv head, kb is the block
+  // within the page (0/1).
+  __device__ __forceinline__ static void load_k(const bf16_t* __restrict__ kpage, int kb, int lane, u32x4 (&kf)[2][DT]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        kf[t][dt] = *reinterpret_cast<const u32x4*>(kpage + ((size_t)((kb * 2 + t) * DT + dt) * 64 + lane) * 8);
+  }
+  __device__ __forceinline__ static void load_v(const bf16_t* __restrict__ vpage, int kb, int lane, u32x4 (&vf)[2 * DT]) {
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t)
+      vf[t] = *reinterpret_cast<const u32x4*>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
+  }
+
+  // One block of 32 keys from loaded fragments; key0 is the absolute position of its first key.  pos[b]:
+  // the position of this lane's query column in tile b (negative: no query).  Keys outside
+  // [pos + 1 - window, pos] are masked.
+  __device__ __forceinline__ void compute(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
+                                          int window, float scale, float cap, int lane) {
     const int g = lane >> 4;
     f32x4 s[NB][2];
 #pragma unroll
@@ -69,11 +84,9 @@ struct Core {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(kpage + ((size_t)((kb * 2 + t) * DT + dt) * 64 + lane) * 8);
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int b = 0; b < NB; ++b) s[b][t] = mfma16(kf, q[b][dt], s[b][t]);
-      }
+        for (int b = 0; b < NB; ++b) s[b][t] = mfma16(kf[t][dt], q[b][dt], s[b][t]);
     u32x4 p[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -112,11 +125,17 @@ struct Core {
       }
     }
 #pragma unroll
-    for (int t = 0; t < 2 * DT; ++t) {
-      const u32x4 vf = *reinterpret_cast<const u32x4*>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
+    for (int t = 0; t < 2 * DT; ++t)
 #pragma unroll
-      for (int b = 0; b < NB; ++b) o[b][t] = mfma16(vf, p[b], o[b][t]);
-    }
+      for (int b = 0; b < NB; ++b) o[b][t] = mfma16(vf[t], p[b], o[b][t]);
+  }
+
+  __device__ __forceinline__ void block32(const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage, int kb,
+                                          int key0, const int* pos, int window, float scale, float cap, int lane) {
+    u32x4 kf[2][DT], vf[2 * DT];
+    load_k(kpage, kb, lane, kf);
+    load_v(vpage, kb, lane, vf);             // in flight while the scores and the softmax are computed
+    compute(kf, vf, key0, pos, window, scale, cap, lane);
   }
 };
 
@@ -223,11 +242,23 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       if (head_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
     }
   }
-  for (int kb32 = my_first; kb32 <= my_last; ++kb32) {
-    const int page = bt[kb32 >> 1];
-    const bf16_t* kp = k_pool + ((size_t)page * nKV + kvh) * page_elems;
-    const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems;
-    c.block32(kp, vp, kb32 & 1, kb32 << 5, cpos, window, scale, cap, lane);
+  // Two sets of fragment registers: while one block of keys is computed, the next one's loads are in flight.
+  {
+    u32x4 kf0[2][DT], vf0[2 * DT], kf1[2][DT], vf1[2 * DT];
+    auto fetch = [&](int kb32, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
+      const int page = bt[kb32 >> 1];
+      Core<DT, 1>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
+      Core<DT, 1>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
+    };
+    if (my_first <= my_last) fetch(my_first, kf0, vf0);
+    for (int kb32 = my_first; kb32 <= my_last; kb32 += 2) {
+      if (kb32 + 1 <= my_last) fetch(kb32 + 1, kf1, vf1);
+      c.compute(kf0, vf0, kb32 << 5, cpos, window, scale, cap, lane);
+      if (kb32 + 1 <= my_last) {
+        if (kb32 + 2 <= my_last) fetch(kb32 + 2, kf0, vf0);
+        c.compute(kf1, vf1, (kb32 + 1) << 5, cpos, window, scale, cap, lane);
+      }
+    }
   }
   // combine the four waves
   if (g == 0) { sm[wave][col] = c.m[0]; sl[wave][col] = c.l[0]; }

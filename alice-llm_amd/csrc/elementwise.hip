@@ -112,6 +112,72 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const float* __restri
     store_f32(o, i, x[i] * inv * (off_pre + load_f32(w_pre, i)));
 }
 
+// The same operation with a row held in registers (EPT elements per thread): every operand is read
+// once and the three phases need no second trip through memory.  Used when the row fits.
+template <typename TW, typename TO, bool FULL, int EPT>
+__global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __restrict__ branch,
+                                     int n_partials, size_t partial_stride,
+                                     const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
+                                     TO* __restrict__ out, const int* __restrict__ rows, int H,
+                                     float eps_post, float eps_pre, float off_post, float off_pre) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t src = (size_t)(rows ? rows[r] : r) * H;
+  float xv[EPT], bv[EPT], wq[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    xv[j] = i < H ? resid[src + i] : 0.f;
+    wq[j] = (w_pre && i < H) ? load_f32(w_pre, i) : 0.f;
+    bv[j] = 0.f;
+  }
+  if (branch) {
+    float wp[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      wp[j] = (w_post && i < H) ? load_f32(w_post, i) : 0.f;
+      if (i < H) {
+        float v = branch[src + i];
+        for (int p = 1; p < n_partials; ++p) v += branch[src + i + p * partial_stride];
+        bv[j] = v;
+      }
+    }
+    if (w_post) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) ss += bv[j] * bv[j];
+      ss = block_sum(ss, red);
+      const float mean = ss / (float)H;
+      const float inv_b = FULL ? 1.f / sqrtf(mean + eps_post) : rsqrtf(mean + eps_post);
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) bv[j] = bv[j] * inv_b * (off_post + wp[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      xv[j] += bv[j];
+      if (i < H) resid[src + i] = xv[j];
+    }
+  }
+  if (!out) return;
+  TO* o = out + (size_t)r * H;
+  float inv = 1.f;
+  if (w_pre) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) ss += xv[j] * xv[j];      // elements beyond H are zero
+    ss = block_sum(ss, red);
+    const float mean = ss / (float)H;
+    inv = FULL ? 1.f / sqrtf(mean + eps_pre) : rsqrtf(mean + eps_pre);
+  }
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < H) store_f32(o, i, w_pre ? xv[j] * inv * (off_pre + wq[j]) : xv[j]);
+  }
+}
+
 extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials, long partial_stride,
                               const void* w_post, const void* w_pre, int w_dtype, void* out, int out_dtype,
                               const int* rows, int T, int H, float eps_post, float eps_pre,
@@ -122,15 +188,26 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
   ALICE_CHECK(!(rows && branch), "add_norm: a row gather cannot be combined with a residual add");
   ALICE_CHECK(n_partials >= 1 && n_partials <= 64, "add_norm: n_partials %d out of range", n_partials);
   if (T == 0) return 0;
-  const int threads = H >= 2048 ? 512 : 256;
+  // Rows up to 8192 wide are held in registers: 256 threads x 1..4 elements, then 1024 threads x 4 or 8.
+  int threads = H >= 2048 ? 512 : 256, ept = 0;
+  if (H <= 1024) { threads = 256; ept = H <= 256 ? 1 : (H <= 512 ? 2 : 4); }
+  else if (H <= 4096) { threads = 1024; ept = 4; }
+  else if (H <= 8192) { threads = 1024; ept = 8; }
+#define ARGS resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, \
+             eps_post, eps_pre, off_post, off_pre
 #define LAUNCH(TW, TO, FULL)                                                                         \
-  add_norm_kernel<TW, TO, FULL><<<T, threads, 0, stream>>>(resid, branch, n_partials,                \
-      (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, eps_post,      \
-      eps_pre, off_post, off_pre)
+  do {                                                                                               \
+    if (ept == 1) add_norm_regs_kernel<TW, TO, FULL, 1><<<T, threads, 0, stream>>>(ARGS);            \
+    else if (ept == 2) add_norm_regs_kernel<TW, TO, FULL, 2><<<T, threads, 0, stream>>>(ARGS);       \
+    else if (ept == 4) add_norm_regs_kernel<TW, TO, FULL, 4><<<T, threads, 0, stream>>>(ARGS);       \
+    else if (ept == 8) add_norm_regs_kernel<TW, TO, FULL, 8><<<T, threads, 0, stream>>>(ARGS);       \
+    else add_norm_kernel<TW, TO, FULL><<<T, threads, 0, stream>>>(ARGS);                             \
+  } while (0)
   DISPATCH_DTYPE(w_dtype, TW, DISPATCH_DTYPE(out_dtype, TO, {
     if (full_precision) LAUNCH(TW, TO, true); else LAUNCH(TW, TO, false);
   }));
 #undef LAUNCH
+#undef ARGS
   ALICE_LAUNCH_CHECK();
   return 0;
 }

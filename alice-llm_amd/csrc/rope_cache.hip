@@ -51,39 +51,30 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
     }
   }
   const int hd2 = d >> 1;        // work items per head: one per pair of the first/second half
-  // q heads and k heads: item = (head, j) with j < d/2 handling elements j and j + d/2 when both lie
-  // in the rotated width, else copying them.
-  const int n_items = (nH + (k_pool ? nKV : 0)) * hd2;
-  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
-    const int h = it / hd2, j = it % hd2;
+  // blockIdx.y names the head this block handles: q heads, then k heads, then v heads.
+  const int h = blockIdx.y;
+  if (h < nH + nKV) {
     const bool is_q = h < nH;
+    if (!is_q && !kdst) return;
     const T* src = row + (size_t)h * d;                     // k heads follow the q heads directly
-    T* dst;
-    if (is_q) dst = q_out + (size_t)t * nH * d + (size_t)h * d;
-    else {
-      if (!kdst) continue;
-      dst = kdst + (size_t)(h - nH) * page_size * d;
-    }
+    T* dst = is_q ? q_out + (size_t)t * nH * d + (size_t)h * d : kdst + (size_t)(h - nH) * page_size * d;
     // where element e goes: q rows are plain; k goes to its place in the page
     auto at = [&](int e) -> size_t { return is_q ? (size_t)e : k_offset(layout, tp, e, d); };
-    // Elements of this item: the rotated pair (j, j + half) if j < half, and the pass-through
-    // elements are handled by the items with j >= half: each copies e = half + j and, when
-    // R < d, nothing is lost because e ranges over [2*half .. ) below.
-    if (j < half) {
-      float x0 = load_f32(src, j), x1 = load_f32(src, j + half);
-      float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
-      store_f32(dst, at(j), x0 * c - x1 * s);
-      store_f32(dst, at(j + half), x0 * s + x1 * c);
+    for (int j = threadIdx.x; j < hd2; j += blockDim.x) {
+      // the rotated pair (j, j + half) if j < half; elements at or beyond R pass through, spread over the items
+      if (j < half) {
+        float x0 = load_f32(src, j), x1 = load_f32(src, j + half);
+        float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
+        store_f32(dst, at(j), x0 * c - x1 * s);
+        store_f32(dst, at(j + half), x0 * s + x1 * c);
+      }
+      for (int e = R + j; e < d; e += hd2) store_f32(dst, at(e), load_f32(src, e));
     }
-    // pass-through elements: indices R .. d-1, spread over the items j of this head
-    for (int e = R + j; e < d; e += hd2) store_f32(dst, at(e), load_f32(src, e));
-  }
-  if (vdst) {
-    const T* vsrc = row + (size_t)(nH + nKV) * d;
-    for (int it = threadIdx.x; it < nKV * d; it += blockDim.x) {
-      const int h = it / d, e = it % d;
-      vdst[(size_t)h * page_size * d + v_offset(layout, tp, e, d)] = vsrc[it];
-    }
+  } else if (vdst) {
+    const int hv = h - nH - nKV;
+    const T* vsrc = row + (size_t)(nH + nKV + hv) * d;
+    T* dst = vdst + (size_t)hv * page_size * d;
+    for (int e = threadIdx.x; e < d; e += blockDim.x) dst[v_offset(layout, tp, e, d)] = vsrc[e];
   }
 }
 
@@ -100,11 +91,12 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
   ALICE_CHECK((k_pool == nullptr) == (v_pool == nullptr), "rope: key and value pools must come together");
   ALICE_CHECK(k_pool == nullptr || (block_table && seq_of_token && page_size > 0 && n_pages > 0 && nKV >= 1),
               "rope: a cache write needs the block table, the token-to-sequence map and the page geometry");
+  ALICE_CHECK(nH + 2 * nKV <= 65535, "rope: too many heads for one launch");
   ALICE_CHECK(row_width >= (nH + (k_pool ? 2 * nKV : 0)) * d, "rope: rows of %d elements are too short for the heads", row_width);
   ALICE_CHECK(kv_layout == 0 || (kv_layout == 1 && page_size == 64 && d % 32 == 0 && dtype == DT_BF16) || k_pool == nullptr,
               "rope: the fragment cache layout needs bfloat16, pages of 64 and head_dim %% 32 == 0");
   if (T == 0) return 0;
-  DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<T, 256, 0, stream>>>(
+  DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<dim3(T, nH + (k_pool ? 2 * nKV : 0)), d >= 256 ? 128 : 64, 0, stream>>>(
       (const TT*)qkv, (TT*)q_out, (TT*)k_pool, (TT*)v_pool, cos_t, sin_t, positions, seq_of_token,
       block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout)));
   ALICE_LAUNCH_CHECK();

@@ -20,15 +20,24 @@ __device__ __forceinline__ uint32_t order_key(float x) {
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
-__global__ __launch_bounds__(ST) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+// Stage 1 (chunks > 1): block (row, chunk) scans its slice of the row and writes (value, index) to `part`;
+// stage 2 runs the same kernel over the partial results.  The lowest index wins among equal values at
+// both stages, so the result does not depend on the number of chunks.
+__global__ __launch_bounds__(ST) void argmax_kernel(const float* __restrict__ vals, const int* __restrict__ idxs,
+                                                    int* __restrict__ out, float* __restrict__ part_v,
+                                                    int* __restrict__ part_i, int V, int chunks) {
   __shared__ float bv[ST / 64];
   __shared__ int bi[ST / 64];
-  const float* row = logits + (size_t)blockIdx.x * V;
+  const float* row = vals + (size_t)blockIdx.x * V;
+  const int* irow = idxs ? idxs + (size_t)blockIdx.x * V : nullptr;
+  const int per = (V + chunks - 1) / chunks;
+  const int lo = blockIdx.y * per, hi = min(V, lo + per);
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += ST) {
+  for (int i = lo + threadIdx.x; i < hi; i += ST) {
     float v = row[i];
-    if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    int id = irow ? irow[i] : i;
+    if (v > best || (v == best && id < idx)) { best = v; idx = id; }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -41,7 +50,12 @@ __global__ __launch_bounds__(ST) void argmax_kernel(const float* __restrict__ lo
   if (threadIdx.x == 0) {
     for (int w = 1; w < ST / 64; ++w)
       if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
-    out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    if (chunks > 1) {
+      part_v[(size_t)blockIdx.x * chunks + blockIdx.y] = best;
+      part_i[(size_t)blockIdx.x * chunks + blockIdx.y] = idx;
+    } else {
+      out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    }
   }
 }
 
@@ -161,10 +175,27 @@ __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ lo
 
 }  // namespace
 
-extern "C" int alice_argmax(const float* logits, int* out, int B, int V, hipStream_t stream) {
+// How many chunks a row is cut into; the workspace holds B * chunks floats and as many ints.
+extern "C" int alice_argmax_chunks(int B, int V) {
+  if (V < 16384) return 1;
+  int c = 512 / (B > 0 ? B : 1);
+  if (c > V / 8192) c = V / 8192;
+  return c < 2 ? 1 : (c > 64 ? 64 : c);
+}
+
+extern "C" int alice_argmax(const float* logits, int* out, float* work_v, int* work_i, int B, int V, hipStream_t stream) {
   ALICE_CHECK(B >= 0 && V >= 1, "argmax: bad sizes B=%d V=%d", B, V);
   if (B == 0) return 0;
-  argmax_kernel<<<B, ST, 0, stream>>>(logits, out, V);
+  const int chunks = alice_argmax_chunks(B, V);
+  ALICE_CHECK(chunks == 1 || (work_v && work_i), "argmax: the workspace is missing");
+  ALICE_CHECK(B <= 65535 * 32, "argmax: too many rows");
+  if (chunks == 1) {
+    argmax_kernel<<<dim3(B, 1), ST, 0, stream>>>(logits, nullptr, out, nullptr, nullptr, V, 1);
+  } else {
+    argmax_kernel<<<dim3(B, chunks), ST, 0, stream>>>(logits, nullptr, out, work_v, work_i, V, chunks);
+    ALICE_LAUNCH_CHECK();
+    argmax_kernel<<<dim3(B, 1), ST, 0, stream>>>(work_v, work_i, out, nullptr, nullptr, chunks, 1);
+  }
   ALICE_LAUNCH_CHECK();
   return 0;
 }

@@ -47,7 +47,8 @@ def _declare(lib) -> None:
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
-        "alice_argmax": [P, P, I, I, P],
+        "alice_argmax": [P, P, P, P, I, I, P],
+        "alice_argmax_chunks": [I, I],
         "alice_sample": [P, P, P, I, I, F, I, F, P],
     }
     for name, args in sigs.items():
@@ -391,7 +392,12 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     if out is None:
         out = torch.empty((B,), dtype=torch.int32, device=logits.device)
     _dev(out, "out", torch.int32, (B,))
-    _call("alice_argmax", logits.data_ptr(), out.data_ptr(), B, V, _stream())
+    chunks = library().alice_argmax_chunks(B, V)
+    wv = wi = None
+    if chunks > 1:
+        wv = torch.empty((B * chunks,), dtype=torch.float32, device=logits.device)
+        wi = torch.empty((B * chunks,), dtype=torch.int32, device=logits.device)
+    _call("alice_argmax", logits.data_ptr(), out.data_ptr(), _opt(wv, "work"), _opt(wi, "work"), B, V, _stream())
     return out
 
 
