@@ -138,8 +138,15 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
       const int i = threadIdx.x + j * blockDim.x;
       wp[j] = (w_post && i < H) ? load_f32(w_post, i) : 0.f;
       if (i < H) {
-        float v = branch[src + i];
-        for (int p = 1; p < n_partials; ++p) v += branch[src + i + p * partial_stride];
+        // partial sums are added in their order; eight loads are in flight at a time
+        float v = 0.f;
+        for (int p0 = 0; p0 < n_partials; p0 += 8) {
+          float t[8];
+#pragma unroll
+          for (int p = 0; p < 8; ++p) t[p] = (p0 + p < n_partials) ? branch[src + i + (size_t)(p0 + p) * partial_stride] : 0.f;
+#pragma unroll
+          for (int p = 0; p < 8; ++p) v += t[p];
+        }
         bv[j] = v;
       }
     }

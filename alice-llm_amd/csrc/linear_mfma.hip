@@ -63,15 +63,15 @@ __device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n
 }
 
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
-// Block: 4 waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + 4, ...; the parts of
-// waves 1..3 go through LDS and wave 0 adds them in the order 1, 2, 3.  grid.x: groups of RT row
+// Block: NW waves on the same RT row tiles; wave w takes runs of k-tiles kb + w U, kb + (w + NW) U, ...;
+// the parts of waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
 // tiles (for GeGLU: RT/2 gate tiles and the RT/2 up tiles that belong to them); grid.y: slices of the
 // inner dimension, each writing its own partial sum y[slice][M][N] (slices > 1 only without epilogue).
-template <int RT, int MT, int EPI, typename TO, bool FULL>
-__global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+template <int RT, int MT, int NW, int EPI, typename TO, bool FULL>
+__global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
                                                             int kt_per_slice, float epi) {
-  extern __shared__ __align__(16) float red[];            // [3][RT*MT][64][4]
+  extern __shared__ __align__(16) float red[];            // [NW - 1][RT*MT][64][4]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int kb = blockIdx.y * kt_per_slice, ke = min(KT, kb + kt_per_slice);
@@ -94,8 +94,8 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __rest
 #pragma unroll
   for (int j = 0; j < MT; ++j) { row[j] = j * 16 + r; row_ok[j] = row[j] < M; }
 
-  constexpr int U = RT >= 4 ? 2 : 4;                      // k-tiles in flight per wave
-  for (int kt0 = kb + wave * U; kt0 < ke; kt0 += 4 * U) {
+  constexpr int U = (RT * MT >= 8) ? 2 : 4;               // k-tiles in flight per wave
+  for (int kt0 = kb + wave * U; kt0 < ke; kt0 += NW * U) {
     u32x4 a[U][RT], b[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __rest
   __syncthreads();
   if (wave != 0) return;
 #pragma unroll
-  for (int w = 0; w < 3; ++w)
+  for (int w = 0; w < NW - 1; ++w)
 #pragma unroll
     for (int i = 0; i < RT; ++i)
 #pragma unroll
@@ -251,6 +251,125 @@ __global__ __launch_bounds__(256) void linear_tiled_mfma_kernel(const bf16_t* __
   }
 }
 
+// ---------------------------------------------------------------- tiled, activations through LDS
+// As above, but the block's 128 tokens x 64 inner elements of activations are staged once in LDS (in
+// fragment order, so LDS reads and writes are linear) and read by all four waves, which cuts the
+// activation traffic from the vector cache by four.  Two stages are kept: while one is used for the
+// MFMAs the next one's global loads are in flight, and one barrier per stage suffices.  The grid is
+// one-dimensional and mapped so that the blocks that share weight tiles run on the same XCD (blocks
+// are dealt to the eight XCDs round robin by their linear index).
+constexpr int KC = 2;      // k-tiles per stage
+
+template <int EPI, typename TO, bool FULL, int TM>
+__global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+                                                               TO* __restrict__ y, int M, int N, int K, int KT, int NT,
+                                                               float epi, int gx, int gy) {
+  constexpr int XJ = TM / 4;                               // token tiles each wave stages
+  __shared__ __align__(16) uint32_t xs_raw[2 * KC * TM * 64 * 4];
+  u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  // Blocks go to the XCDs round robin by index; XCD x works through the x-th eighth of the tiles in
+  // column-major order, so that tiles with the same weight columns meet in one L2.
+  const int id = blockIdx.x, xcd = id & 7, local = id >> 3;
+  const int per = (gx * gy + 7) >> 3;
+  const int item = xcd * per + local;
+  if (local >= per || item >= gx * gy) return;
+  const int bx = item / gy, by = item % gy;
+  const int m0 = by * (16 * TM);
+  int tile[WN];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) {
+    if (EPI == ALICE_EPI_GEGLU) {
+      const int pair = (bx * 4 + wave) * (WN / 2) + (i >> 1);
+      tile[i] = (i & 1) ? N / 16 + pair : pair;
+      if (pair >= N / 16) tile[i] = NT;
+    } else {
+      tile[i] = (bx * 4 + wave) * WN + i;
+    }
+  }
+  int xrow[XJ];
+#pragma unroll
+  for (int j = 0; j < XJ; ++j) xrow[j] = min(m0 + (XJ * wave + j) * 16 + r, M - 1);
+
+  f32x4 acc[WN][TM];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 xr[KC][XJ], wk[KC][WN];
+  auto stage_load = [&](int s) {
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+      for (int j = 0; j < XJ; ++j) xr[kc][j] = load_x_frag(x, xrow[j], true, K, s * KC + kc, g);
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+      for (int j = 0; j < XJ; ++j) xs[((buf * KC + kc) * TM + XJ * wave + j) * 64 + lane] = xr[kc][j];
+  };
+  auto w_load = [&](int kt, u32x4 (&w)[WN]) {
+#pragma unroll
+    for (int i = 0; i < WN; ++i) {
+      w[i] = u32x4{0u, 0u, 0u, 0u};
+      if (tile[i] < NT && kt < KT) w[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
+    }
+  };
+  const int S = (KT + KC - 1) / KC;
+  stage_load(0);
+  stage_store(0);
+#pragma unroll
+  for (int kc = 0; kc < KC; ++kc) w_load(kc, wk[kc]);
+  for (int s = 0; s < S; ++s) {
+    if (s + 1 < S) stage_load(s + 1);
+    __syncthreads();
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      u32x4 xf[TM];
+#pragma unroll
+      for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC + kc) * TM + j) * 64 + lane];
+#pragma unroll
+      for (int i = 0; i < WN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
+      // this k-tile's weight registers are free again: fetch the same slot of the next stage
+      if (s + 1 < S) w_load((s + 1) * KC + kc, wk[kc]);
+    }
+    if (s + 1 < S) stage_store((s + 1) & 1);
+  }
+
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = m0 + j * 16 + r;
+    if (m >= M) continue;
+    const size_t row_off = (size_t)m * N;
+    if (EPI == ALICE_EPI_GEGLU) {
+#pragma unroll
+      for (int p = 0; p < WN / 2; ++p) {
+        if (tile[2 * p] >= NT) continue;
+        const int n = tile[2 * p] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
+        store4(y, row_off, n, N, o);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < WN; ++i) {
+        if (tile[i] >= NT) continue;
+        const int n = tile[i] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
+        store4(y, row_off, n, N, o);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- layout conversion
 __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N, int K, int KT, size_t total) {
   const size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x;     // index in dst, in elements
@@ -272,24 +391,34 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   const int groups = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, RT / 2) : ceil_div(NT, RT);
   const int per = ceil_div(KT, split);
   dim3 grid(groups, split);
-  const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-  linear_skinny_kernel<RT, MT, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+  // Eight waves a block when the slice is long enough to give each of them work and the block count is
+  // too low to fill the chip with four.
+  const bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
+  if (eight) {
+    const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
+    linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+  } else {
+    const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
+    linear_skinny_kernel<RT, MT, 4, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+  }
   ALICE_LAUNCH_CHECK();
   return 0;
 }
 
 // Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
 // on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)
-int skinny_row_tiles(int N, int epi) {
+int skinny_row_tiles(int M, int N, int epi) {
   const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   if (tiles >= 4096) return 4;
+  if (M > 32 && tiles >= 1024) return 4;          // many tokens: more rows per block per read of the activations
+  if (M > 32 && tiles >= 256) return 2;
   if (tiles >= 1024 || epi == ALICE_EPI_GEGLU) return 2;
   return 1;
 }
 
 template <int EPI, typename TO>
 int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
-  const int rt = skinny_row_tiles(N, EPI);
+  const int rt = skinny_row_tiles(M, N, EPI);
 #define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, s)
 #define BY_RT(MT)                                                   \
   do {                                                              \
@@ -305,12 +434,27 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
   return 1;
 }
 
+int g_tiled_variant = 0;     // 0: activations through LDS; 1: every wave loads its own (for comparison)
+
 template <int EPI, typename TO>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, float epi, hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
-  dim3 grid(gx, ceil_div(M, 16 * WM));
-  linear_tiled_mfma_kernel<EPI, TO, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi);
+  int gy = ceil_div(M, 16 * WM);
+  if (g_tiled_variant == 0) {
+    // 128 tokens a block, or 64 when that leaves the chip less than full
+    if (gx * gy >= 384 || M <= 64) {
+      const int blocks = 8 * ceil_div(gx * gy, 8);
+      linear_tiled_lds_kernel<EPI, TO, false, 8><<<blocks, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy);
+    } else {
+      gy = ceil_div(M, 64);
+      const int blocks = 8 * ceil_div(gx * gy, 8);
+      linear_tiled_lds_kernel<EPI, TO, false, 4><<<blocks, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy);
+    }
+  } else {
+    dim3 grid(gx, gy);
+    linear_tiled_mfma_kernel<EPI, TO, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi);
+  }
   ALICE_LAUNCH_CHECK();
   return 0;
 }
@@ -318,6 +462,7 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, flo
 }  // namespace
 
 extern "C" int alice_has_mfma_linear() { return 1; }
+extern "C" void alice_set_tiled_variant(int v) { g_tiled_variant = v; }
 
 // Whether a matrix of `rows` x K with this epilogue can use the fragment layout.
 extern "C" int alice_frag16_supported(int rows, int K, int epilogue) {
@@ -338,7 +483,7 @@ extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStre
 int alice_linear_split_hint_frag(int M, int N, int K) {
   if (M > 64) return 1;
   const int KT = (K + 31) / 32;
-  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(N, ALICE_EPI_NONE));
+  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE));
   int split = 1;
   // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
   while (groups * split < 1024 && KT / (split * 2) >= 16 && split < 16) split *= 2;
