@@ -27,9 +27,23 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)f32_to_bf16(a).bits | ((uint32_t)f32_to_bf16(b).bits << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // one instruction; exp2(-inf) = 0
+__device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+// Constants of the score pipeline.  A raw dot product s becomes, in the base-2 domain in which the
+// softmax runs (2^y = e^score):
+//   with softcap:  y = cap log2e tanh(s scale / cap),  tanh(x) = 1 - 2 / (2^(2 log2e x) + 1)
+//   without:       y = s scale log2e
+struct ScoreConsts {
+  float c_in, c_out;
+  __device__ __forceinline__ ScoreConsts(float scale, float cap) {
+    if (cap > 0.f) { c_in = scale / cap * 2.f * LOG2E; c_out = cap * LOG2E; }
+    else { c_in = scale * LOG2E; c_out = 0.f; }
+  }
+};
 // max / sum over the four lanes that hold the same query column (l, l^16, l^32, l^48)
 __device__ __forceinline__ float col_max(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, 64));
@@ -73,10 +87,12 @@ struct Core {
   }
 
   // One block of 32 keys from loaded fragments; key0 is the absolute position of its first key.  pos[b]:
-  // the position of this lane's query column in tile b (negative: no query).  Keys outside
-  // [pos + 1 - window, pos] are masked.
+  // the position of this lane's query column in tile b (negative: no query).  With EDGE, keys outside
+  // [pos + 1 - window, pos] are masked; the caller passes EDGE = false only for blocks that every query
+  // of the wave sees whole.  The running maximum m and the scores are kept in the base-2 domain.
+  template <bool SOFTCAP, bool EDGE>
   __device__ __forceinline__ void compute(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
-                                          int window, float scale, float cap, int lane) {
+                                          int window, ScoreConsts k, int lane) {
     const int g = lane >> 4;
     f32x4 s[NB][2];
 #pragma unroll
@@ -96,22 +112,24 @@ struct Core {
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = key0 + t * 16 + g * 4 + i;
-          float v = s[b][t][i] * scale;
-          if (cap > 0.f) v = cap * tanh_fast(v / cap);
-          v = (key <= pos[b] && key >= lo) ? v : -INFINITY;
+          float v = s[b][t][i] * k.c_in;
+          if (SOFTCAP) v = fmaf(-2.f * k.c_out, rcp_fast(exp2_fast(v) + 1.f), k.c_out);
+          if (EDGE) {
+            const int key = key0 + t * 16 + g * 4 + i;
+            v = (key <= pos[b] && key >= lo) ? v : -INFINITY;
+          }
           s[b][t][i] = v;
           mx = fmaxf(mx, v);
         }
       const float m_new = fmaxf(m[b], col_max(mx));
-      const float corr = (m[b] == -INFINITY) ? 0.f : __expf(m[b] - m_new);       // m_new >= m[b]
-      const float base = (m_new == -INFINITY) ? 0.f : m_new;                    // all masked so far: p = exp(-inf) = 0
+      const float base = (m_new == -INFINITY) ? 0.f : m_new;                    // all masked so far: every p is 0
+      const float corr = exp2_fast(m[b] - base);                                // m[b] = -inf gives 0
       float sum = 0.f;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = __expf(s[b][t][i] - base);
+          const float e = exp2_fast(s[b][t][i] - base);
           s[b][t][i] = e;
           sum += e;
         }
@@ -130,19 +148,20 @@ struct Core {
       for (int b = 0; b < NB; ++b) o[b][t] = mfma16(vf[t], p[b], o[b][t]);
   }
 
-  __device__ __forceinline__ void block32(const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage, int kb,
-                                          int key0, const int* pos, int window, float scale, float cap, int lane) {
-    u32x4 kf[2][DT], vf[2 * DT];
-    load_k(kpage, kb, lane, kf);
-    load_v(vpage, kb, lane, vf);             // in flight while the scores and the softmax are computed
-    compute(kf, vf, key0, pos, window, scale, cap, lane);
+  // Masked or whole block.
+  template <bool SOFTCAP>
+  __device__ __forceinline__ void compute_any(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
+                                              int window, ScoreConsts k, bool edge, int lane) {
+    // (Two instantiations, masked and unmasked, cost more registers than the mask's few instructions save.)
+    (void)edge;
+    compute<SOFTCAP, true>(kf, vf, key0, pos, window, k, lane);
   }
 };
 
 // ---------------------------------------------------------------- prompts
 // grid: (tiles of 64 query tokens, sequences, kv heads); 4 waves, wave w takes tokens 16 w .. 16 w + 15
 // of the tile for GH query heads at a time (both share the kv head), looping over the group's heads.
-template <int DT, int GH>
+template <int DT, int GH, bool SOFTCAP>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
@@ -163,6 +182,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int* bt = block_table + (size_t)b * bt_stride;
   const int group = nH / nKV;
   const size_t page_elems = (size_t)64 * D;
+  const ScoreConsts sc(scale, cap);
 
   for (int h0 = 0; h0 < group; h0 += GH) {
     Core<DT, GH> c;
@@ -180,11 +200,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         if (ok) c.q[hh][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
       }
     }
+    // A block of keys is whole for this wave if every one of its queries sees all 32 keys.
+    const int whole_until = start_len + first - 31;              // key0 <= this: no query is before the block's end
+    const int whole_from = window > 0 ? last_pos + 1 - window : 0;   // key0 >= this: no query's window starts inside
+    u32x4 kf[2][DT], vf[2 * DT];
     for (int kb32 = first_key >> 5; kb32 <= (last_pos >> 5); ++kb32) {
       const int page = bt[kb32 >> 1];
-      const bf16_t* kp = k_pool + ((size_t)page * nKV + kvh) * page_elems;
-      const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems;
-      c.block32(kp, vp, kb32 & 1, kb32 << 5, pos, window, scale, cap, lane);
+      Core<DT, GH>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
+      Core<DT, GH>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);   // in flight during the scores
+      const int key0 = kb32 << 5;
+      const bool edge = key0 > whole_until || key0 < whole_from;
+      c.template compute_any<SOFTCAP>(kf, vf, key0, pos, window, sc, edge, lane);
     }
 #pragma unroll
     for (int hh = 0; hh < GH; ++hh) {
@@ -208,7 +234,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // splits * 4 waves; every wave keeps a running (max, sum, output); the block's four waves are combined
 // in LDS in the order 0, 1, 2, 3 and the split's result goes to `parts`:
 // [sequence][head][split][D + 2] = (max, sum, unnormalised output).  With one split the output is final.
-template <int DT>
+template <int DT, bool SOFTCAP>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, float* __restrict__ parts, const int* __restrict__ context_lens,
@@ -232,6 +258,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
   Core<DT, 1> c;
   c.init();
+  const ScoreConsts sc(scale, cap);
   const bool head_ok = col < group;
   int cpos[1] = {head_ok ? pos : -1};
   {
@@ -253,10 +280,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     if (my_first <= my_last) fetch(my_first, kf0, vf0);
     for (int kb32 = my_first; kb32 <= my_last; kb32 += 2) {
       if (kb32 + 1 <= my_last) fetch(kb32 + 1, kf1, vf1);
-      c.compute(kf0, vf0, kb32 << 5, cpos, window, scale, cap, lane);
+      c.template compute_any<SOFTCAP>(kf0, vf0, kb32 << 5, cpos, window, sc, kb32 == kb_first || kb32 == kb_last, lane);
       if (kb32 + 1 <= my_last) {
         if (kb32 + 2 <= my_last) fetch(kb32 + 2, kf0, vf0);
-        c.compute(kf1, vf1, (kb32 + 1) << 5, cpos, window, scale, cap, lane);
+        c.template compute_any<SOFTCAP>(kf1, vf1, (kb32 + 1) << 5, cpos, window, sc, kb32 + 1 == kb_last, lane);
       }
     }
   }
@@ -276,7 +303,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     float acc = 0.f, ll = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float f = (sm[w][hc] == -INFINITY) ? 0.f : __expf(sm[w][hc] - mm);
+      const float f = (sm[w][hc] == -INFINITY) ? 0.f : exp2_fast(sm[w][hc] - mm);     // maxima are base-2 exponents
       acc += so[((size_t)w * group + hc) * (D + 4) + e] * f;
       ll += sl[w][hc] * f;
     }
@@ -300,7 +327,7 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
     float acc = 0.f, ll = 0.f;
     for (int s = 0; s < splits; ++s) {
       const float* ps = pr + (size_t)s * (D + 2);
-      const float f = (ps[0] == -INFINITY) ? 0.f : __expf(ps[0] - mm);
+      const float f = (ps[0] == -INFINITY) ? 0.f : exp2_fast(ps[0] - mm);
       acc += ps[2 + e] * f;
       ll += ps[1] * f;
     }
@@ -325,8 +352,15 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   if (B == 0 || max_new == 0) return 0;
   dim3 grid(ceil_div(max_new, 64), B, nKV);
   const int group = nH / nKV;
-#define GO(DT, GH) attn_prefill_kernel<DT, GH><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-      (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window)
+#define GO(DT, GH)                                                                                                          \
+  do {                                                                                                                      \
+    if (softcap > 0.f)                                                                                                      \
+      attn_prefill_kernel<DT, GH, true><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+    else                                                                                                                    \
+      attn_prefill_kernel<DT, GH, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+  } while (0)
   if (d == 64) { if (group % 2 == 0) GO(2, 2); else GO(2, 1); }
   else if (d == 128) { if (group % 2 == 0) GO(4, 2); else GO(4, 1); }
   else { if (group % 2 == 0) GO(8, 2); else GO(8, 1); }
@@ -353,8 +387,15 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
   if (B == 0) return 0;
   dim3 grid(B, nKV, splits);
   const size_t lds = (size_t)4 * (nH / nKV) * (d + 4) * sizeof(float);
-#define GO(DT) attn_decode_kernel<DT><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-      (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits)
+#define GO(DT)                                                                                                              \
+  do {                                                                                                                      \
+    if (softcap > 0.f)                                                                                                      \
+      attn_decode_kernel<DT, true><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits);              \
+    else                                                                                                                    \
+      attn_decode_kernel<DT, false><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits);              \
+  } while (0)
   if (d == 64) GO(2); else if (d == 128) GO(4); else GO(8);
 #undef GO
   ALICE_LAUNCH_CHECK();

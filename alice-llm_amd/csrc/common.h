@@ -20,17 +20,18 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
   return __uint_as_float(bits16 << 16);
 }
-// Round to nearest even; NaN stays NaN.
+// Round to nearest even; NaN stays NaN (the hardware conversion of gfx950).
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r.bits = (uint16_t)((u >> 16) | 0x0040u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (uint16_t)(u >> 16);
-  }
+  r.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
   return r;
+}
+// Two values rounded and packed, the first in the low half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p, size_t i);
@@ -90,10 +91,10 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 // tanh at full precision for the 32-bit path, a fast form for the bfloat16 path.
 __device__ __forceinline__ float tanh_full(float x) { return tanhf(x); }
 __device__ __forceinline__ float tanh_fast(float x) {
-  // tanh(x) = 1 - 2 / (exp(2x) + 1); the clamp keeps exp finite.  Relative error about 1e-6.
-  float xc = fminf(fmaxf(x, -15.f), 15.f);
-  float e = __expf(2.f * xc);
-  return 1.f - 2.f / (e + 1.f);
+  // tanh(x) = 1 - 2 / (2^(2 log2e x) + 1) with the hardware's exp2 and reciprocal (about 1 ulp each):
+  // absolute error about 2e-7; 2^x overflows to +inf and underflows to 0, which give exactly +-1.
+  float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
+  return fmaf(-2.f, __builtin_amdgcn_rcpf(e + 1.f), 1.f);
 }
 __device__ __forceinline__ float gelu_tanh_f(float z, bool full) {
   float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);

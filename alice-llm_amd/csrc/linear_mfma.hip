@@ -50,8 +50,8 @@ __device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n
     if constexpr (sizeof(TO) == 4) {
       *reinterpret_cast<f32x4*>((float*)y + row_off + n) = v;
     } else {
-      uint32_t lo = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
-      uint32_t hi = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+      uint32_t lo = pack_bf16x2(v[0], v[1]);
+      uint32_t hi = pack_bf16x2(v[2], v[3]);
       uint2 pk = {lo, hi};
       *reinterpret_cast<uint2*>((bf16_t*)y + row_off + n) = pk;
     }
