@@ -63,8 +63,8 @@ __device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n
 }
 
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
-// Block: NW waves on the same RT row tiles; wave w takes runs of k-tiles kb + w U, kb + (w + NW) U, ...;
-// the parts of waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
+// Block: NW waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + NW, ...; the parts of
+// waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
 // tiles (for GeGLU: RT/2 gate tiles and the RT/2 up tiles that belong to them); grid.y: slices of the
 // inner dimension, each writing its own partial sum y[slice][M][N] (slices > 1 only without epilogue).
 template <int RT, int MT, int NW, int EPI, typename TO, bool FULL>
@@ -94,28 +94,42 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
 #pragma unroll
   for (int j = 0; j < MT; ++j) { row[j] = j * 16 + r; row_ok[j] = row[j] < M; }
 
-  constexpr int U = (RT * MT >= 8) ? 2 : 4;               // k-tiles in flight per wave
-  for (int kt0 = kb + wave * U; kt0 < ke; kt0 += NW * U) {
-    u32x4 a[U][RT], b[U][MT];
+  // A rolling window of U k-tiles per wave: wave w takes k-tiles kb + w, kb + w + NW, ...; as soon as a
+  // tile's fragments have gone into the MFMAs their registers are refilled with the tile U steps ahead,
+  // so U loads per operand stay in flight all the time.
+  constexpr int U = (RT * MT >= 8) ? 3 : 4;
+  u32x4 a[U][RT], b[U][MT];
+  auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
+    const bool kok = kt < ke;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kt = kt0 + u;
-      const bool kok = kt < ke;
-#pragma unroll
-      for (int i = 0; i < RT; ++i) {
-        a[u][i] = u32x4{0u, 0u, 0u, 0u};
-        if (kok && tile[i] < tile_limit)
-          a[u][i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
-      }
-#pragma unroll
-      for (int j = 0; j < MT; ++j) b[u][j] = load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
+    for (int i = 0; i < RT; ++i) {
+      aa[i] = u32x4{0u, 0u, 0u, 0u};
+      if (kok && tile[i] < tile_limit)
+        aa[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int j = 0; j < MT; ++j) bb[j] = load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
+  };
+  // Blocks start at different places of their k range and wrap around: all blocks read the same
+  // activations, and in lockstep they would all ask the same L2 channel for the same line at once.
+  const int J = (ke - kb + NW - 1) / NW;                    // k-tiles per wave (the last ones may be past the end)
+  const int rot = J > 0 ? (int)(blockIdx.x % (unsigned)J) : 0;
+  auto tile_at = [&](int t) {                               // t-th tile of this wave's rotated sequence
+    int j = t + rot;
+    if (j >= J) j -= J;
+    return t < J ? kb + wave + j * NW : ke;                 // past the sequence: nothing to load
+  };
+#pragma unroll
+  for (int u = 0; u < U; ++u) fetch(tile_at(u), a[u], b[u]);
+  for (int t0 = 0; t0 < J; t0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < MT; ++j) acc[i][j] = mfma16(a[u][i], b[u][j], acc[i][j]);
+      fetch(tile_at(t0 + U + u), a[u], b[u]);      // tiles past the end come back as zeros
+    }
   }
 
   if (wave > 0) {
@@ -385,6 +399,8 @@ __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restr
   dst[o] = (n < N && k < K) ? src[(size_t)n * K + k] : z;
 }
 
+int g_skinny_rt = 0, g_skinny_nw = 0;      // tuning overrides (0: choose by shape)
+
 template <int RT, int MT, int EPI, typename TO>
 int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
@@ -393,7 +409,8 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   dim3 grid(groups, split);
   // Eight waves a block when the slice is long enough to give each of them work and the block count is
   // too low to fill the chip with four.
-  const bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
+  bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
+  if (g_skinny_nw) eight = g_skinny_nw == 8 && RT * MT <= 8;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
     linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
@@ -407,18 +424,20 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
 
 // Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
 // on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)
-int skinny_row_tiles(int M, int N, int epi) {
+int skinny_row_tiles(int M, int N, int epi, int split) {
+  if (g_skinny_rt) return g_skinny_rt;
   const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   if (tiles >= 4096) return 4;
-  if (M > 32 && tiles >= 1024) return 4;          // many tokens: more rows per block per read of the activations
-  if (M > 32 && tiles >= 256) return 2;
+  // Many tokens: more rows per block per read of the activations, wherever the inner dimension can be
+  // split over blocks to keep the chip busy (measured on the 2B shapes).
+  if (M > 32 && (tiles >= 1024 || (split > 1 && tiles >= 64))) return 4;
   if (tiles >= 1024 || epi == ALICE_EPI_GEGLU) return 2;
   return 1;
 }
 
 template <int EPI, typename TO>
 int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
-  const int rt = skinny_row_tiles(M, N, EPI);
+  const int rt = skinny_row_tiles(M, N, EPI, split);
 #define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, s)
 #define BY_RT(MT)                                                   \
   do {                                                              \
@@ -463,6 +482,7 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, flo
 
 extern "C" int alice_has_mfma_linear() { return 1; }
 extern "C" void alice_set_tiled_variant(int v) { g_tiled_variant = v; }
+extern "C" void alice_set_skinny_override(int row_tiles, int waves) { g_skinny_rt = row_tiles; g_skinny_nw = waves; }
 
 // Whether a matrix of `rows` x K with this epilogue can use the fragment layout.
 extern "C" int alice_frag16_supported(int rows, int K, int epilogue) {
@@ -483,7 +503,8 @@ extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStre
 int alice_linear_split_hint_frag(int M, int N, int K) {
   if (M > 64) return 1;
   const int KT = (K + 31) / 32;
-  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE));
+  if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);
+  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE, 1));
   int split = 1;
   // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
   while (groups * split < 1024 && KT / (split * 2) >= 16 && split < 16) split *= 2;
@@ -499,7 +520,9 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f, "linear: softcap must be positive");
   ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0, "linear: operands must be 16-byte aligned");
   if (M == 0) return 0;
-  bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64);
+  // Up to 64 tokens stream the weights once; very wide matrices (the output head) have enough column
+  // blocks for the tiled kernel, which shares the activations through LDS, as soon as there are 17 tokens.
+  bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 16 && N >= 65536 && split_k == 1));
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
   ALICE_CHECK(split_k == 1 || (skinny && epi == ALICE_EPI_NONE && y_dtype == DT_F32),
               "linear: partial sums need the streaming kernel, no epilogue and float32 output");

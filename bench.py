@@ -2,9 +2,10 @@
 
     python bench.py --gpus 1 --steps K --warmup W
 
-A step is one decode step of a batch of 8 sequences that were prefilled with 2,048-token prompts
-(context length 4,096 in the cache).  The printed line also holds the prefill of one 2,048-token
-prompt, the decode step's memory roofline, and decode throughput at batch 1 and 64.
+A step is one decode step of a batch of 8 sequences that were prefilled with 2,048-token prompts;
+by default the timed steps run the context from 2,048 out to 4,096.  The printed line also holds the
+prefill of one 2,048-token prompt, the decode step's memory roofline (at the mean context of the timed
+steps), and decode throughput at batch 1 and 64 over the same range.
 """
 import argparse
 import json
@@ -43,7 +44,7 @@ def prefill_flops(cfg, T, n_logit_rows=1):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--steps", type=int, default=2048)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--preset", default="2b")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the preset (both numbers are reported)")
@@ -52,7 +53,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure decode at ('' for none)")
-    ap.add_argument("--point-steps", type=int, default=64)
+    ap.add_argument("--point-steps", type=int, default=None, help="steps for the other batch sizes (default: --steps)")
     ap.add_argument("--no-prefill", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -84,7 +85,8 @@ def main() -> int:
     def decode_run(batch, steps, warmup):
         """Prefill `batch` prompts, then time `steps` decode steps (greedy, tokens fed back)."""
         from alice_llm_amd.hip import ops
-        eng = model.engine(max_tokens=batch * args.context, max_seqs=batch)
+        per_seq = -(-(args.prompt + warmup + steps) // 64) * 64
+        eng = model.engine(max_tokens=batch * max(args.context, per_seq), max_seqs=batch)
         slots = eng.open(batch)
         ps = prompts(batch)
         chunk = max(1, 16384 // args.prompt)                 # prefill a few sequences at a time
@@ -138,8 +140,9 @@ def main() -> int:
     achieved = nbytes / (ms_step / 1e3) / 1e9
     points = {}
     for b in [int(x) for x in args.points.split(",") if x]:
-        pdt, _, _ = decode_run(b, args.point_steps, min(args.warmup, 4))
-        points[f"decode_b{b}"] = round(b * args.point_steps / pdt, 1)
+        psteps = args.point_steps or args.steps
+        pdt, _, _ = decode_run(b, psteps, args.warmup)
+        points[f"decode_b{b}"] = round(b * psteps / pdt, 1)
         print(f"[bench] decode_b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
