@@ -507,3 +507,15 @@ def test_attention_mfma_refuses_other_head_sizes():
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     with pytest.raises(ops.HipLibraryError, match="head_dim 96 is not covered"):
         ops.attention_decode(q, kp, kp, q.clone(), i32([5]), i32([[1]]), num_heads=1, max_context=5, scale=1.0, softcap=None, window=None)
+
+
+def test_linear_mfma_vocabulary_sized_output():
+    # the output head's shape: a quarter of a million rows, a width that is no power of two
+    N, K = 256000, 96
+    w = rnd(N, K, seed=40, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    for M in (1, 8, 64, 100):
+        x = rnd(M, K, seed=41, dtype=torch.bfloat16)
+        y = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_SOFTCAP, epi_param=30.0, full_precision=False)
+        close(y, 30.0 * torch.tanh((x.double() @ w.double().T) / 30.0), 2e-3)
