@@ -44,14 +44,20 @@ struct ScoreConsts {
     else { c_in = scale * LOG2E; c_out = 0.f; }
   }
 };
-// max / sum over the four lanes that hold the same query column (l, l^16, l^32, l^48)
+// max / sum over the four lanes that hold the same query column (l, l^16, l^32, l^48), with gfx950's
+// lane-swap instructions: permlane32_swap(v, v) gives (value of the lane's copy in the lower half, in
+// the upper half), permlane16_swap(v, v) the same for the even and odd rows of 16 lanes.
 __device__ __forceinline__ float col_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 16, 64));
-  return fmaxf(v, __shfl_xor(v, 32, 64));
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float col_sum(float v) {
-  v += __shfl_xor(v, 16, 64);
-  return v + __shfl_xor(v, 32, 64);
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);                 // the same two addends in the same order in every lane
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // Running state of NB query tiles (16 query columns each) against the keys seen so far.
@@ -86,27 +92,31 @@ struct Core {
       vf[t] = *reinterpret_cast<const u32x4*>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
   }
 
-  // One block of 32 keys from loaded fragments; key0 is the absolute position of its first key.  pos[b]:
-  // the position of this lane's query column in tile b (negative: no query).  With EDGE, keys outside
-  // [pos + 1 - window, pos] are masked; the caller passes EDGE = false only for blocks that every query
-  // of the wave sees whole.  The running maximum m and the scores are kept in the base-2 domain.
-  template <bool SOFTCAP, bool EDGE>
-  __device__ __forceinline__ void compute(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
-                                          int window, ScoreConsts k, int lane) {
+  // Scores of one block of 32 keys from loaded key fragments; key0 is the absolute position of its first
+  // key.  pos[b]: the position of this lane's query column in tile b (negative: no query).  Keys outside
+  // [pos + 1 - window, pos] are masked.  Updates the running maximum (base-2 domain, common to the four
+  // lanes of a column), rescales the output, adds to this lane's own share of the running sum (the lanes
+  // of a column are added up once, in finish()), and returns the probabilities as the second operand of
+  // the value product.
+  template <bool SOFTCAP>
+  __device__ __forceinline__ void scores(const u32x4 (&kf)[2][DT], int key0, const int* pos, int window, ScoreConsts k,
+                                         int lane, u32x4 (&p)[NB]) {
     const int g = lane >> 4;
     f32x4 s[NB][2];
 #pragma unroll
     for (int b = 0; b < NB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int b = 0; b < NB; ++b) s[b][t] = mfma16(kf[t][dt], q[b][dt], s[b][t]);
-    u32x4 p[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      const int lo = window > 0 ? pos[b] + 1 - window : 0;
+      // key visible iff lo <= key <= pos, i.e. (unsigned)(key - lo) <= (unsigned)(pos - lo); no query: span 0 and rel > 0
+      const int lo = window > 0 ? max(pos[b] + 1 - window, 0) : 0;
+      const unsigned span = pos[b] >= 0 ? (unsigned)(pos[b] - lo) : 0u;
+      const int rel0 = pos[b] >= 0 ? key0 + g * 4 - lo : 1 << 30;
       float mx = -INFINITY;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -114,10 +124,7 @@ struct Core {
         for (int i = 0; i < 4; ++i) {
           float v = s[b][t][i] * k.c_in;
           if (SOFTCAP) v = fmaf(-2.f * k.c_out, rcp_fast(exp2_fast(v) + 1.f), k.c_out);
-          if (EDGE) {
-            const int key = key0 + t * 16 + g * 4 + i;
-            v = (key <= pos[b] && key >= lo) ? v : -INFINITY;
-          }
+          v = ((unsigned)(rel0 + t * 16 + i) <= span) ? v : -INFINITY;
           s[b][t][i] = v;
           mx = fmaxf(mx, v);
         }
@@ -133,7 +140,7 @@ struct Core {
           s[b][t][i] = e;
           sum += e;
         }
-      l[b] = l[b] * corr + col_sum(sum);
+      l[b] = l[b] * corr + sum;
       m[b] = m_new;
       p[b] = u32x4{pack2(s[b][0][0], s[b][0][1]), pack2(s[b][0][2], s[b][0][3]),
                    pack2(s[b][1][0], s[b][1][1]), pack2(s[b][1][2], s[b][1][3])};
@@ -142,10 +149,29 @@ struct Core {
         for (int t = 0; t < 2 * DT; ++t) o[b][t] *= corr;
       }
     }
+  }
+
+  // Adds the value product of output tiles [t0, t0 + N) from their loaded fragments.
+  template <int N>
+  __device__ __forceinline__ void accumulate(const u32x4 (&vf)[N], int t0, const u32x4 (&p)[NB]) {
 #pragma unroll
-    for (int t = 0; t < 2 * DT; ++t)
+    for (int t = 0; t < N; ++t)
 #pragma unroll
-      for (int b = 0; b < NB; ++b) o[b][t] = mfma16(vf[t], p[b], o[b][t]);
+      for (int b = 0; b < NB; ++b) o[b][t0 + t] = mfma16(vf[t], p[b], o[b][t0 + t]);
+  }
+
+  template <bool SOFTCAP, bool EDGE>
+  __device__ __forceinline__ void compute(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
+                                          int window, ScoreConsts k, int lane) {
+    u32x4 p[NB];
+    scores<SOFTCAP>(kf, key0, pos, window, k, lane, p);
+    accumulate<2 * DT>(vf, 0, p);
+  }
+
+  // The lanes of a column hold shares of its running sum: add them up (same order in every lane).
+  __device__ __forceinline__ void finish() {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) l[b] = col_sum(l[b]);
   }
 
   // Masked or whole block.
@@ -159,19 +185,25 @@ struct Core {
 };
 
 // ---------------------------------------------------------------- prompts
-// grid: (tiles of 64 query tokens, sequences, kv heads); 4 waves, wave w takes tokens 16 w .. 16 w + 15
-// of the tile for GH query heads at a time (both share the kv head), looping over the group's heads.
+// grid: (tiles of 64 query tokens, sequences, kv heads x passes); 4 waves, wave w takes tokens
+// 16 w .. 16 w + 15 of the tile for GH query heads of one kv head (a pass); the passes of a kv head's
+// group are separate blocks.  Tiles are taken from the end of the prompt backwards: the last tiles see
+// the most keys, and starting them first shortens the tail.  With one head per wave (GH = 1) there are
+// registers for two sets of key/value fragments, and the next block's loads fly during the current
+// block's arithmetic.
 template <int DT, int GH, bool SOFTCAP>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
     const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
   constexpr int D = DT * 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, g = lane >> 4;
-  const int b = blockIdx.y, kvh = blockIdx.z;
+  const int group = nH / nKV, passes = (group + GH - 1) / GH;
+  const int b = blockIdx.y, kvh = blockIdx.z / passes, h0 = (blockIdx.z % passes) * GH;
   const int t_begin = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_begin;
-  const int first = blockIdx.x * 64 + wave * 16;            // this wave's first token within the sequence's new tokens
+  const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int first = tile * 64 + wave * 16;                  // this wave's first token within the sequence's new tokens
   if (first >= n_new) return;
   const int start_len = context_lens[b] - n_new;
   const int my_tok = first + col;
@@ -180,51 +212,157 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int last_pos = start_len + min(first + 15, n_new - 1);
   const int first_key = window > 0 ? max(0, start_len + first + 1 - window) : 0;
   const int* bt = block_table + (size_t)b * bt_stride;
-  const int group = nH / nKV;
   const size_t page_elems = (size_t)64 * D;
   const ScoreConsts sc(scale, cap);
 
-  for (int h0 = 0; h0 < group; h0 += GH) {
-    Core<DT, GH> c;
-    c.init();
-    int pos[GH];
+  Core<DT, GH> c;
+  c.init();
+  int pos[GH];
 #pragma unroll
-    for (int hh = 0; hh < GH; ++hh) {
-      const int head = kvh * group + h0 + hh;
-      const bool ok = tok_ok && (h0 + hh) < group;
-      pos[hh] = ok ? my_pos : -1;
-      const bf16_t* qrow = q + ((size_t)(t_begin + (tok_ok ? my_tok : 0)) * nH + (ok ? head : kvh * group)) * D;
+  for (int hh = 0; hh < GH; ++hh) {
+    const int head = kvh * group + h0 + hh;
+    const bool ok = tok_ok && (h0 + hh) < group;
+    pos[hh] = ok ? my_pos : -1;
+    const bf16_t* qrow = q + ((size_t)(t_begin + (tok_ok ? my_tok : 0)) * nH + (ok ? head : kvh * group)) * D;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        c.q[hh][dt] = u32x4{0u, 0u, 0u, 0u};
-        if (ok) c.q[hh][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
-      }
+    for (int dt = 0; dt < DT; ++dt) {
+      c.q[hh][dt] = u32x4{0u, 0u, 0u, 0u};
+      if (ok) c.q[hh][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
     }
-    // A block of keys is whole for this wave if every one of its queries sees all 32 keys.
-    const int whole_until = start_len + first - 31;              // key0 <= this: no query is before the block's end
-    const int whole_from = window > 0 ? last_pos + 1 - window : 0;   // key0 >= this: no query's window starts inside
-    u32x4 kf[2][DT], vf[2 * DT];
-    for (int kb32 = first_key >> 5; kb32 <= (last_pos >> 5); ++kb32) {
+  }
+  // A block of keys is whole for this wave if every one of its queries sees all 32 keys.
+  const int whole_until = start_len + first - 31;              // key0 <= this: no query is before the block's end
+  const int whole_from = window > 0 ? last_pos + 1 - window : 0;   // key0 >= this: no query's window starts inside
+  const int kb_begin = first_key >> 5, kb_end = last_pos >> 5;
+  auto fetch = [&](int kb32, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
+    const int page = bt[kb32 >> 1];
+    Core<DT, GH>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
+    Core<DT, GH>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
+  };
+  auto edge_of = [&](int kb32) { return (kb32 << 5) > whole_until || (kb32 << 5) < whole_from; };
+  if constexpr (GH == 1) {
+    // Two waves per SIMD (256 registers each) hide each other's waits.  Keys and the first half of the values
+    // are fetched together; the second half of the values goes into the registers that the keys leave.
+    for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
       const int page = bt[kb32 >> 1];
+      const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems + ((size_t)(kb32 & 1) * 2 * DT * 64 + lane) * 8;
+      u32x4 kf[2][DT], va[DT], vb[DT], p[1];
       Core<DT, GH>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
-      Core<DT, GH>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);   // in flight during the scores
-      const int key0 = kb32 << 5;
-      const bool edge = key0 > whole_until || key0 < whole_from;
-      c.template compute_any<SOFTCAP>(kf, vf, key0, pos, window, sc, edge, lane);
-    }
 #pragma unroll
-    for (int hh = 0; hh < GH; ++hh) {
-      if (pos[hh] < 0) continue;
-      const int head = kvh * group + h0 + hh;
-      const float inv = 1.f / c.l[hh];
-      bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
+      for (int t = 0; t < DT; ++t) va[t] = *reinterpret_cast<const u32x4*>(vp + (size_t)t * 512);
+      c.template scores<SOFTCAP>(kf, kb32 << 5, pos, window, sc, lane, p);
 #pragma unroll
-      for (int t = 0; t < 2 * DT; ++t) {
-        const f32x4 v = c.o[hh][t] * inv;
-        uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
-        *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
-      }
+      for (int t = 0; t < DT; ++t) vb[t] = *reinterpret_cast<const u32x4*>(vp + (size_t)(DT + t) * 512);
+      c.template accumulate<DT>(va, 0, p);
+      c.template accumulate<DT>(vb, DT, p);
     }
+  } else {
+    u32x4 kf[2][DT], vf[2 * DT];
+    for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
+      fetch(kb32, kf, vf);                                       // the values are in flight during the scores
+      c.template compute_any<SOFTCAP>(kf, vf, kb32 << 5, pos, window, sc, edge_of(kb32), lane);
+    }
+  }
+  c.finish();
+#pragma unroll
+  for (int hh = 0; hh < GH; ++hh) {
+    if (pos[hh] < 0) continue;
+    const int head = kvh * group + h0 + hh;
+    const float inv = 1.f / c.l[hh];
+    bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t) {
+      const f32x4 v = c.o[hh][t] * inv;
+      uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+      *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+    }
+  }
+}
+
+// Prompts, second form: a block of four waves takes one tile of 16 query tokens of one head and the waves
+// split its keys into four contiguous runs, as the single-token kernel below does; the parts are
+// combined in LDS in the order 0, 1, 2, 3.  A single long prompt then gives thousands of short waves
+// instead of a few hundred long ones, which is what fills the chip.
+// grid: (tiles of 16 query tokens, taken from the end backwards; sequences; query heads).
+template <int DT, bool SOFTCAP>
+__global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
+  constexpr int D = DT * 32;
+  __shared__ float sm[4][16], sl[4][16];
+  extern __shared__ __align__(16) float so[];                // [3 waves][16 columns][D + 4]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int group = nH / nKV;
+  const int b = blockIdx.y, head = blockIdx.z, kvh = head / group;
+  const int t_begin = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_begin;
+  const int first = ((int)gridDim.x - 1 - (int)blockIdx.x) * 16;
+  if (first >= n_new) return;                                // the whole block
+  const int start_len = context_lens[b] - n_new;
+  const int my_tok = first + col;
+  const bool tok_ok = my_tok < n_new;
+  int pos[1] = {tok_ok ? start_len + my_tok : -1};
+  const int last_pos = start_len + min(first + 15, n_new - 1);
+  const int first_key = window > 0 ? max(0, start_len + first + 1 - window) : 0;
+  const int kb_first = first_key >> 5, kb_last = last_pos >> 5;
+  const int per = (kb_last - kb_first + 4) / 4;              // ceil(blocks / 4)
+  const int my_first = kb_first + wave * per, my_last = min(kb_last, my_first + per - 1);
+  const int* bt = block_table + (size_t)b * bt_stride;
+  const size_t page_elems = (size_t)64 * D;
+  const ScoreConsts sc(scale, cap);
+
+  Core<DT, 1> c;
+  c.init();
+  {
+    const bf16_t* qrow = q + ((size_t)(t_begin + (tok_ok ? my_tok : 0)) * nH + head) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      c.q[0][dt] = u32x4{0u, 0u, 0u, 0u};
+      if (tok_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
+    }
+  }
+  for (int kb32 = my_first; kb32 <= my_last; ++kb32) {
+    const int page = bt[kb32 >> 1];
+    const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems + ((size_t)(kb32 & 1) * 2 * DT * 64 + lane) * 8;
+    u32x4 kf[2][DT], va[DT], vb[DT], p[1];
+    Core<DT, 1>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) va[t] = *reinterpret_cast<const u32x4*>(vp + (size_t)t * 512);
+    c.template scores<SOFTCAP>(kf, kb32 << 5, pos, window, sc, lane, p);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) vb[t] = *reinterpret_cast<const u32x4*>(vp + (size_t)(DT + t) * 512);   // into the keys' registers
+    c.template accumulate<DT>(va, 0, p);
+    c.template accumulate<DT>(vb, DT, p);
+  }
+  c.finish();
+  if (g == 0) { sm[wave][col] = c.m[0]; sl[wave][col] = c.l[0]; }
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t)
+      *reinterpret_cast<f32x4*>(&so[((size_t)(wave - 1) * 16 + col) * (D + 4) + t * 16 + g * 4]) = c.o[0][t];
+  }
+  __syncthreads();
+  if (wave != 0 || !tok_ok) return;
+  // wave 0 adds the parts of waves 1..3 to its own, each scaled to the common maximum
+  float mm = fmaxf(fmaxf(sm[0][col], sm[1][col]), fmaxf(sm[2][col], sm[3][col]));
+  float f[4], ll = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    f[w] = (sm[w][col] == -INFINITY) ? 0.f : exp2_fast(sm[w][col] - mm);
+    ll += sl[w][col] * f[w];
+  }
+  const float inv = 1.f / ll;
+  bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
+#pragma unroll
+  for (int t = 0; t < 2 * DT; ++t) {
+    f32x4 v = c.o[0][t] * f[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+      v += *reinterpret_cast<const f32x4*>(&so[((size_t)(w - 1) * 16 + col) * (D + 4) + t * 16 + g * 4]) * f[w];
+    v *= inv;
+    uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+    *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
   }
 }
 
@@ -288,6 +426,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
   }
   // combine the four waves
+  c.finish();
   if (g == 0) { sm[wave][col] = c.m[0]; sl[wave][col] = c.l[0]; }
   if (head_ok) {
 #pragma unroll
@@ -337,6 +476,10 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
 
 }  // namespace
 
+int g_prefill_variant = 0;     // 0: chosen by the grid's size; 1: whole tiles per wave; 2: keys split over a block's waves
+int g_prefill_heads = 0;       // 0: heads per wave chosen by the grid's size; 1 or 2 force it
+extern "C" void alice_set_prefill_variant(int v, int heads) { g_prefill_variant = v; g_prefill_heads = heads; }
+
 // Head sizes the matrix-core kernels and the fragment cache layout cover.
 extern "C" int alice_attention_mfma_supported(int d) { return d == 64 || d == 128 || d == 256; }
 
@@ -350,8 +493,13 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   ALICE_CHECK(B >= 0 && max_new >= 0 && B <= 65535 && nKV <= 65535, "attention: bad batch B=%d", B);
   ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
   if (B == 0 || max_new == 0) return 0;
-  dim3 grid(ceil_div(max_new, 64), B, nKV);
   const int group = nH / nKV;
+  // Two heads a wave halve the key/value reads.
+  const long waves2 = (long)ceil_div(max_new, 64) * B * nKV * ceil_div(group, 2) * 4;
+  int gh = group % 2 == 0 ? 2 : 1;
+  if (g_prefill_heads == 1 || (g_prefill_heads == 2 && group % 2 == 0)) gh = g_prefill_heads;
+  ALICE_CHECK((long)nKV * ceil_div(group, gh) <= 65535, "attention: too many heads for one launch");
+  dim3 grid(ceil_div(max_new, 64), B, nKV * ceil_div(group, gh));
 #define GO(DT, GH)                                                                                                          \
   do {                                                                                                                      \
     if (softcap > 0.f)                                                                                                      \
@@ -361,9 +509,29 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
       attn_prefill_kernel<DT, GH, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
           (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
   } while (0)
-  if (d == 64) { if (group % 2 == 0) GO(2, 2); else GO(2, 1); }
-  else if (d == 128) { if (group % 2 == 0) GO(4, 2); else GO(4, 1); }
-  else { if (group % 2 == 0) GO(8, 2); else GO(8, 1); }
+#define GOS(DT)                                                                                                             \
+  do {                                                                                                                      \
+    dim3 sgrid(ceil_div(max_new, 16), B, nH);                                                                               \
+    const size_t lds = (size_t)3 * 16 * (DT * 32 + 4) * sizeof(float);                                                      \
+    if (softcap > 0.f)                                                                                                      \
+      attn_prefill_split_kernel<DT, true><<<sgrid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+    else                                                                                                                    \
+      attn_prefill_split_kernel<DT, false><<<sgrid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+  } while (0)
+  // Few waves (one prompt of a few thousand tokens): split every tile's keys over four waves.  Many: whole
+  // tiles per wave, two heads a wave where the group is even.
+  const bool split = g_prefill_variant == 2 || (g_prefill_variant == 0 && waves2 < 4096);
+  if (split) {
+    ALICE_CHECK(nH <= 65535, "attention: too many heads for one launch");
+    if (d == 64) GOS(2); else if (d == 128) GOS(4); else GOS(8);
+  } else {
+    if (d == 64) { if (gh == 2) GO(2, 2); else GO(2, 1); }
+    else if (d == 128) { if (gh == 2) GO(4, 2); else GO(4, 1); }
+    else { if (gh == 2) GO(8, 2); else GO(8, 1); }
+  }
+#undef GOS
 #undef GO
   ALICE_LAUNCH_CHECK();
   return 0;

@@ -340,15 +340,18 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
   for (int s = 0; s < S; ++s) {
     if (s + 1 < S) stage_load(s + 1);
     __syncthreads();
+    u32x4 xf[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC) * TM + j) * 64 + lane];
 #pragma unroll
     for (int kc = 0; kc < KC; ++kc) {
-      u32x4 xf[TM];
 #pragma unroll
-      for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC + kc) * TM + j) * 64 + lane];
+      for (int j = 0; j < TM; ++j) {
 #pragma unroll
-      for (int i = 0; i < WN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
+        for (int i = 0; i < WN; ++i) acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
+        // this token tile's fragment has had its last use: read the next k-tile's into the same registers
+        if (kc + 1 < KC) xf[j] = xs[(((s & 1) * KC + kc + 1) * TM + j) * 64 + lane];
+      }
       // this k-tile's weight registers are free again: fetch the same slot of the next stage
       if (s + 1 < S) w_load((s + 1) * KC + kc, wk[kc]);
     }
