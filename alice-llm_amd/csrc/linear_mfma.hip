@@ -277,7 +277,7 @@ constexpr int KC = 2;      // k-tiles per stage
 template <int EPI, typename TO, bool FULL, int TM>
 __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                               float epi, int gx, int gy) {
+                                                               float epi, int gx, int gy, int kt_per_slice) {
   constexpr int XJ = TM / 4;                               // token tiles each wave stages
   __shared__ __align__(16) uint32_t xs_raw[2 * KC * TM * 64 * 4];
   u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
@@ -313,11 +313,12 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
     for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   u32x4 xr[KC][XJ], wk[KC][WN];
+  const int kt_base = blockIdx.y * kt_per_slice, kt_end = min(KT, kt_base + kt_per_slice);
   auto stage_load = [&](int s) {
 #pragma unroll
     for (int kc = 0; kc < KC; ++kc)
 #pragma unroll
-      for (int j = 0; j < XJ; ++j) xr[kc][j] = load_x_frag(x, xrow[j], true, K, s * KC + kc, g);
+      for (int j = 0; j < XJ; ++j) xr[kc][j] = load_x_frag(x, xrow[j], kt_base + s * KC + kc < kt_end, K, kt_base + s * KC + kc, g);
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
@@ -325,14 +326,18 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
 #pragma unroll
       for (int j = 0; j < XJ; ++j) xs[((buf * KC + kc) * TM + XJ * wave + j) * 64 + lane] = xr[kc][j];
   };
-  auto w_load = [&](int kt, u32x4 (&w)[WN]) {
+  auto w_load = [&](int rel, u32x4 (&w)[WN]) {                // rel: k-tile relative to the slice
+    const int kt = kt_base + rel;
 #pragma unroll
     for (int i = 0; i < WN; ++i) {
       w[i] = u32x4{0u, 0u, 0u, 0u};
-      if (tile[i] < NT && kt < KT) w[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
+      if (tile[i] < NT && kt < kt_end) w[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
     }
   };
-  const int S = (KT + KC - 1) / KC;
+  // blockIdx.y: the slice of the inner dimension this block sums (its own partial result y[slice][M][N])
+  const int kt_lo = blockIdx.y * kt_per_slice, kt_hi = min(KT, kt_lo + kt_per_slice);
+  const int S = (kt_hi - kt_lo + KC - 1) / KC;
+  y += (size_t)blockIdx.y * M * N;
   stage_load(0);
   stage_store(0);
 #pragma unroll
@@ -459,19 +464,20 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
 int g_tiled_variant = 0;     // 0: activations through LDS; 1: every wave loads its own (for comparison)
 
 template <int EPI, typename TO>
-int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, float epi, hipStream_t s) {
+int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
   if (g_tiled_variant == 0) {
     // 128 tokens a block, or 64 when that leaves the chip less than full
-    if (gx * gy >= 384 || M <= 64) {
-      const int blocks = 8 * ceil_div(gx * gy, 8);
-      linear_tiled_lds_kernel<EPI, TO, false, 8><<<blocks, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy);
+    const int per = ceil_div(KT, split);
+    if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
+      dim3 grid(8 * ceil_div(gx * gy, 8), split);
+      linear_tiled_lds_kernel<EPI, TO, false, 8><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
     } else {
       gy = ceil_div(M, 64);
-      const int blocks = 8 * ceil_div(gx * gy, 8);
-      linear_tiled_lds_kernel<EPI, TO, false, 4><<<blocks, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy);
+      dim3 grid(8 * ceil_div(gx * gy, 8), split);
+      linear_tiled_lds_kernel<EPI, TO, false, 4><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
     }
   } else {
     dim3 grid(gx, gy);
@@ -504,7 +510,13 @@ extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStre
 }
 
 int alice_linear_split_hint_frag(int M, int N, int K) {
-  if (M > 64) return 1;
+  if (M > 64) {
+    // Tiled kernel: 128 tokens x 256 features a block.  Narrow outputs leave most of the chip idle: halve
+    // or quarter the inner dimension instead of the tile.
+    const int blocks = ceil_div(N, 256) * ceil_div(M, 128), KT = (K + 31) / 32;
+    if (blocks >= 200 || KT < 32) return 1;
+    return (blocks < 200 && KT >= 256) ? 4 : 2;
+  }
   const int KT = (K + 31) / 32;
   if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);
   const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE, 1));
@@ -527,8 +539,8 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   // blocks for the tiled kernel, which shares the activations through LDS, as soon as there are 17 tokens.
   bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 16 && N >= 65536 && split_k == 1));
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
-  ALICE_CHECK(split_k == 1 || (skinny && epi == ALICE_EPI_NONE && y_dtype == DT_F32),
-              "linear: partial sums need the streaming kernel, no epilogue and float32 output");
+  ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && (skinny || g_tiled_variant == 0)),
+              "linear: partial sums need no epilogue and float32 output");
   ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
 #define BY_EPI(FN, ...)                                                                            \
   do {                                                                                             \
@@ -543,6 +555,6 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
     }                                                                                              \
   } while (0)
   if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, stream);
-  BY_EPI(launch_tiled, x, w, y, M, N, K, epi_param, stream);
+  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, stream);
 #undef BY_EPI
 }
