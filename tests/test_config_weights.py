@@ -135,3 +135,19 @@ def test_random_weights_folder():
     assert torch.equal(a["model.embed_tokens.weight"], src32.tensor("model.embed_tokens.weight"))
     b = dict(random_tensors(specs, 2, torch.float32))
     assert not torch.equal(a["model.norm.weight"], b["model.norm.weight"])
+
+
+def test_sharded_folder(tmp_path):
+    from safetensors.torch import save_file
+    a = {"x.weight": torch.randn(4, 3).bfloat16()}
+    b = {"y.weight": torch.randn(5)}
+    save_file(a, str(tmp_path / "model-00001-of-00002.safetensors"))
+    save_file(b, str(tmp_path / "model-00002-of-00002.safetensors"))
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {
+        "x.weight": "model-00001-of-00002.safetensors", "y.weight": "model-00002-of-00002.safetensors"}}))
+    src = TensorSource(str(tmp_path))
+    assert sorted(src.keys()) == ["x.weight", "y.weight"] and torch.equal(src.tensor("y.weight"), b["y.weight"])
+    assert src.info("x.weight") == (torch.bfloat16, (4, 3))
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"x.weight": "missing.safetensors"}}))
+    with pytest.raises(WeightFileError, match="missing.safetensors"):
+        TensorSource(str(tmp_path))

@@ -202,3 +202,36 @@ def test_captured_decode_steps_match_eager_on_every_replay(name, dtype):
     got = torch.cat([graph.step(s, [[t]], "last").clone() for t in seqs[3][500:]])
     assert max_err(got, ref[500:]) < tol(dtype, ref)
     graph.cache.check_consistent()
+
+
+@pytest.mark.parametrize("name,dtype", [("tiny-b", "float32"), ("tiny-c", "bfloat16"), ("tiny-c", "float32")])
+def test_stale_cache_contents_and_slot_order_change_nothing(name, dtype):
+    """Pages are handed out again without being cleared.  Here every page of every pool is first filled with
+    huge values: a kernel that read one position beyond a sequence's length, or before its window, would
+    show it.  The same requests are then run in another slot order; logits are bitwise the same."""
+    model, plain = setup(name, dtype)
+    eng = model.engine(max_tokens=64 * 12, max_seqs=4, use_graphs=False)
+    for g in eng.cache.groups:
+        g.k.fill_(1e30)
+        g.v.fill_(-1e30)
+    seqs = [random_tokens(plain.V, n, 70 + i) for i, n in enumerate((100, 33, 65))]
+    refs = [plain.forward(s) for s in seqs]
+
+    def run(order):
+        slots = eng.open(4)                       # one slot stays unused; its number shifts the others
+        use = [slots[i] for i in order]
+        a = eng.step(use, [s[:-2] for s in seqs], "all")
+        b = eng.step(use, [[s[-2]] for s in seqs], "last")
+        c = eng.step(use, [[s[-1]] for s in seqs], "last")
+        eng.close(slots)
+        return a, b, c
+
+    a, b, c = run([0, 1, 2])
+    ref_a = torch.cat([r[:-2] for r in refs])
+    assert max_err(a, ref_a) < tol(dtype, ref_a)
+    assert max_err(b, torch.stack([r[-2] for r in refs])) < tol(dtype, ref_a)
+    assert max_err(c, torch.stack([r[-1] for r in refs])) < tol(dtype, ref_a)
+    a2, b2, c2 = run([3, 0, 2])                   # other slots, other pages (the free list has been reshuffled)
+    assert torch.equal(a, a2) and torch.equal(b, b2) and torch.equal(c, c2)
+    a3, b3, c3 = run([3, 0, 2])                   # and run to run
+    assert torch.equal(a2, a3) and torch.equal(c2, c3)

@@ -322,3 +322,71 @@ def test_toy_architecture_against_its_plain_replica():
     got = torch.cat([eng.step(s, [toks[:9]], "all")] + [eng.step(s, [[t]], "last") for t in toks[9:]])
     ref = toy_plain(model, toks)
     assert (got.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("prec", PRECS)
+def test_embedding_and_tied_head_parts(prec):
+    from alice_llm_amd.parts import EMBEDDINGS, HEADS
+    p = Precision.of(prec)
+    V, H = 203, 72
+    emb = EMBEDDINGS.get("embedding")(p, vocab_size=V, dim=H, scale=2.5)
+    head = HEADS.get("lm_head")(p, vocab_size=V, dim=H, softcap=4.0, tied_to="emb")
+    assert head.param_specs() == {} and emb.param_specs()["weight"].shape == (V, H)
+    E = rnd(V, H, seed=30, scale=0.3, dtype=torch.bfloat16)
+    emb.assign("weight", E)
+    emb.finalize(); head.finalize(); head.tie(emb)
+    tok = torch.tensor([0, 202, 17, 17], dtype=torch.int32, device=DEV)
+    x = emb.forward(tok)
+    assert x.dtype == torch.float32 and (x.double() - E.double()[tok.long()] * 2.5).abs().max() < 1e-6
+    n = rnd(5, H, seed=31, dtype=p.act)
+    logits = head.forward(n)
+    ref = 4.0 * torch.tanh((n.double() @ E.double().T) / 4.0)
+    assert logits.dtype == torch.float32 and (logits.double() - ref).abs().max() < tol(prec)
+    untied = HEADS.get("lm_head")(p, vocab_size=V, dim=H, softcap=None, tied_to=None)
+    assert untied.param_specs()["weight"].shape == (V, H)
+    untied.assign("weight", E)
+    assert (untied.forward(n).double() - n.double() @ E.double().T).abs().max() < tol(prec) * 3
+
+
+def test_rotary_part_table_is_accurate_far_out():
+    p = Precision.of("float32")
+    rope = POSITIONS.get("rope")(p, DEV, dim=256, theta=10000.0, max_positions=8192)
+    j = torch.arange(128, dtype=D)
+    ang = 8191.0 * 10000.0 ** (-2.0 * j / 256)
+    assert (rope.cos[8191].double().cpu() - torch.cos(ang)).abs().max() < 1e-7      # 64-bit angles, rounded once
+    # the same angles taken in 32-bit, as the reference does (llama3.rs:5367-5378), are off by up to 5e-4 here
+    ang32 = (torch.tensor(8191.0) * (1.0 / torch.tensor(10000.0).pow(2.0 * torch.arange(128.0) / 256))).double()
+    assert (torch.cos(ang32) - torch.cos(ang)).abs().max() < 1e-3
+    with pytest.raises(ValueError, match="rotated width"):
+        POSITIONS.get("rope")(p, DEV, dim=16, theta=1e4, max_positions=8, rotary_dim=18)
+
+
+def test_block_part_with_toy_parts_and_an_unfused_norm():
+    """The block arrangement alone: toy mixer/feed-forward that scale their input, a norm the stream cannot
+    fuse (no `fused` method), and the pre-norm-only form."""
+    p = Precision.of("float32")
+
+    class Scale:
+        def __init__(self, f): self.f = f
+        def forward(self, x, ctx, cache=None): return (x.float() * self.f).contiguous()
+
+    class PlainLayerNorm:                       # no fused(): the stream runs it through forward()
+        def forward(self, x, out_dtype, rows=None):
+            x = x if rows is None else x.index_select(0, rows.long())
+            return torch.nn.functional.layer_norm(x, x.shape[-1:]).to(out_dtype)
+
+    ln = PlainLayerNorm()
+    x0 = rnd(7, 40, seed=33, scale=2.0)
+    blk = BLOCKS.get("sandwich")(Scale(0.5), Scale(-0.25), {"pre_mixer": ln, "post_mixer": ln, "pre_ff": ln, "post_ff": None})
+    s = ResidualStream(x0.clone(), p)
+    blk.forward(s, None, None)
+    s.flush()
+    LN = lambda t: torch.nn.functional.layer_norm(t, t.shape[-1:])
+    x1 = x0 + LN(0.5 * LN(x0))
+    x2 = x1 - 0.25 * LN(x1)
+    assert (s.x - x2).abs().max() < 1e-5
+    pre = BLOCKS.get("prenorm")(Scale(2.0), Scale(1.0), {})          # no norms at all: x + 2x, then + that
+    s = ResidualStream(x0.clone(), p)
+    pre.forward(s, None, None)
+    s.flush()
+    assert (s.x - 6.0 * x0).abs().max() < 1e-4
