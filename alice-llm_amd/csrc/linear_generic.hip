@@ -98,6 +98,79 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
   }
 }
 
+// Up to 8 tokens: one wave per output feature streams that feature's weight row once (coalesced, four
+// elements a lane a step) against all the tokens' activations; the lanes' partial sums meet in a fixed
+// shuffle tree, so a token's result does not depend on the others.  For GeGLU the wave takes the gate
+// row and the up row of its feature.
+template <typename TA, typename TW, typename TO, int EPI, bool FULL, int MB>
+__global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                          TO* __restrict__ Y, int M, int N, int K, float epi) {
+  const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  constexpr int NR = EPI == ALICE_EPI_GEGLU ? 2 : 1;
+  float acc[NR][MB];
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[r][m] = 0.f;
+  const int K4 = K & ~3;
+  for (int k = lane * 4; k < K4; k += 256) {
+    float w[NR][4];
+#pragma unroll
+    for (int r = 0; r < NR; ++r)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[r][e] = load_f32(W, (size_t)(n + r * N) * K + k + e);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      if (m < M) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float xv = load_f32(A, (size_t)m * K + k + e);
+#pragma unroll
+          for (int r = 0; r < NR; ++r) acc[r][m] = fmaf(w[r][e], xv, acc[r][m]);
+        }
+      }
+    }
+  }
+  if (lane < K - K4) {                                       // up to three columns beyond the last whole group of four
+    const int k = K4 + lane;
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+      if (m < M) {
+        const float xv = load_f32(A, (size_t)m * K + k);
+#pragma unroll
+        for (int r = 0; r < NR; ++r) acc[r][m] = fmaf(load_f32(W, (size_t)(n + r * N) * K + k), xv, acc[r][m]);
+      }
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    if (m >= M) continue;
+    float v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) v[r] = wave_sum(acc[r][m]);
+    if (lane == 0) {
+      float o = v[0];
+      if (EPI == ALICE_EPI_GEGLU) o = gelu_tanh_f(v[0], FULL) * v[NR - 1];
+      if (EPI == ALICE_EPI_SOFTCAP) o = epi * (FULL ? tanh_full(o / epi) : tanh_fast(o / epi));
+      store_f32(Y, (size_t)m * N + n, o);
+    }
+  }
+}
+
+template <typename TA, typename TW, typename TO, bool FULL>
+int launch_rows(const void* x, const void* w, void* y, int M, int N, int K, int epi, float epi_param, hipStream_t stream) {
+  const int grid = ceil_div(N, 4);
+#define GO(E, MB) linear_rows_kernel<TA, TW, TO, E, FULL, MB><<<grid, 256, 0, stream>>>((const TA*)x, (const TW*)w, (TO*)y, M, N, K, epi_param)
+#define BY_M(E) do { if (M <= 1) GO(E, 1); else if (M <= 2) GO(E, 2); else if (M <= 4) GO(E, 4); else GO(E, 8); } while (0)
+  if (epi == ALICE_EPI_NONE) BY_M(ALICE_EPI_NONE);
+  else if (epi == ALICE_EPI_GEGLU) BY_M(ALICE_EPI_GEGLU);
+  else BY_M(ALICE_EPI_SOFTCAP);
+#undef BY_M
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
 template <typename TA, typename TW, typename TO, bool FULL>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int epi, float epi_param,
                  hipStream_t stream) {
@@ -124,9 +197,14 @@ int alice_linear_generic(const void* x, int x_dtype, const void* w, int w_dtype,
   ALICE_CHECK(ceil_div(M, BM) <= 65535, "linear: M=%d has too many row tiles for one launch", M);
   if (M == 0) return 0;
   int rc = 0;
+  const bool rows = M <= 8 && N >= 64;                       // few tokens: stream each weight row once
   DISPATCH_DTYPE(x_dtype, TA, DISPATCH_DTYPE(w_dtype, TW, DISPATCH_DTYPE(y_dtype, TO, {
-    rc = full_precision ? launch_tiled<TA, TW, TO, true>(x, w, y, M, N, K, epi, epi_param, stream)
-                        : launch_tiled<TA, TW, TO, false>(x, w, y, M, N, K, epi, epi_param, stream);
+    if (rows)
+      rc = full_precision ? launch_rows<TA, TW, TO, true>(x, w, y, M, N, K, epi, epi_param, stream)
+                          : launch_rows<TA, TW, TO, false>(x, w, y, M, N, K, epi, epi_param, stream);
+    else
+      rc = full_precision ? launch_tiled<TA, TW, TO, true>(x, w, y, M, N, K, epi, epi_param, stream)
+                          : launch_tiled<TA, TW, TO, false>(x, w, y, M, N, K, epi, epi_param, stream);
   })));
   return rc;
 }

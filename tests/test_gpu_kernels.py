@@ -86,7 +86,7 @@ def test_softcap():
 
 
 # ------------------------------------------------------------------ matrix product
-LINEAR_SHAPES = [(1, 96, 64), (7, 200, 144), (64, 130, 320), (65, 64, 33), (300, 97, 100)]
+LINEAR_SHAPES = [(1, 96, 64), (7, 200, 144), (8, 70, 37), (3, 63, 64), (64, 130, 320), (65, 64, 33), (300, 97, 100)]
 
 
 @pytest.mark.parametrize("M,N,K", LINEAR_SHAPES)
@@ -105,7 +105,7 @@ def test_linear_generic(M, N, K, xdt, wdt, ydt):
     close(y2, 2.0 * torch.tanh(ref / 2.0), 1e-5 if full else 5e-4)
 
 
-@pytest.mark.parametrize("M,N,K", [(3, 48, 64), (70, 160, 96), (9, 33, 40)])
+@pytest.mark.parametrize("M,N,K", [(3, 48, 64), (70, 160, 96), (9, 33, 40), (8, 128, 70), (1, 320, 96)])
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_linear_generic_geglu(M, N, K, dt):
     x, w = rnd(M, K, seed=8, dtype=DT[dt]), rnd(2 * N, K, seed=9, scale=0.3, dtype=DT[dt])
