@@ -13,6 +13,10 @@
 #define ALICE_LAYOUT_ROW 0     // row-major [N, K]
 #define ALICE_LAYOUT_FRAG16 1  // bfloat16 in 16x32 MFMA fragments, see linear_mfma.hip
 
+#define ALICE_PREFILL_AUTO 0    // prompt attention: chosen by the grid's size
+#define ALICE_PREFILL_TILES 1   // a wave takes whole tiles of 16 queries (two heads where the group is even)
+#define ALICE_PREFILL_SPLIT 2   // the four waves of a block split one tile's keys
+
 #define ALICE_LINEAR_AUTO 0
 #define ALICE_LINEAR_GENERIC 1
 #define ALICE_LINEAR_SKINNY 2
@@ -68,7 +72,7 @@ int alice_attention_mfma_supported(int d);
 int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
                             const int* cu_seqlens, const int* context_lens, const int* block_table,
                             int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
-                            float scale, float softcap, int window, hipStream_t stream);
+                            float scale, float softcap, int window, int variant, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                            const int* context_lens, const int* block_table, int bt_stride, int B, int nH,

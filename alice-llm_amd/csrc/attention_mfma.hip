@@ -160,7 +160,7 @@ struct Core {
       for (int b = 0; b < NB; ++b) o[b][t0 + t] = mfma16(vf[t], p[b], o[b][t0 + t]);
   }
 
-  template <bool SOFTCAP, bool EDGE>
+  template <bool SOFTCAP>
   __device__ __forceinline__ void compute(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
                                           int window, ScoreConsts k, int lane) {
     u32x4 p[NB];
@@ -172,15 +172,6 @@ struct Core {
   __device__ __forceinline__ void finish() {
 #pragma unroll
     for (int b = 0; b < NB; ++b) l[b] = col_sum(l[b]);
-  }
-
-  // Masked or whole block.
-  template <bool SOFTCAP>
-  __device__ __forceinline__ void compute_any(const u32x4 (&kf)[2][DT], const u32x4 (&vf)[2 * DT], int key0, const int* pos,
-                                              int window, ScoreConsts k, bool edge, int lane) {
-    // (Two instantiations, masked and unmasked, cost more registers than the mask's few instructions save.)
-    (void)edge;
-    compute<SOFTCAP, true>(kf, vf, key0, pos, window, k, lane);
   }
 };
 
@@ -230,16 +221,12 @@ __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
       if (ok) c.q[hh][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
     }
   }
-  // A block of keys is whole for this wave if every one of its queries sees all 32 keys.
-  const int whole_until = start_len + first - 31;              // key0 <= this: no query is before the block's end
-  const int whole_from = window > 0 ? last_pos + 1 - window : 0;   // key0 >= this: no query's window starts inside
   const int kb_begin = first_key >> 5, kb_end = last_pos >> 5;
   auto fetch = [&](int kb32, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
     const int page = bt[kb32 >> 1];
     Core<DT, GH>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
     Core<DT, GH>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
   };
-  auto edge_of = [&](int kb32) { return (kb32 << 5) > whole_until || (kb32 << 5) < whole_from; };
   if constexpr (GH == 1) {
     // Two waves per SIMD (256 registers each) hide each other's waits.  Keys and the first half of the values
     // are fetched together; the second half of the values goes into the registers that the keys leave.
@@ -260,7 +247,7 @@ __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
     u32x4 kf[2][DT], vf[2 * DT];
     for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
       fetch(kb32, kf, vf);                                       // the values are in flight during the scores
-      c.template compute_any<SOFTCAP>(kf, vf, kb32 << 5, pos, window, sc, edge_of(kb32), lane);
+      c.template compute<SOFTCAP>(kf, vf, kb32 << 5, pos, window, sc, lane);
     }
   }
   c.finish();
@@ -418,10 +405,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     if (my_first <= my_last) fetch(my_first, kf0, vf0);
     for (int kb32 = my_first; kb32 <= my_last; kb32 += 2) {
       if (kb32 + 1 <= my_last) fetch(kb32 + 1, kf1, vf1);
-      c.template compute_any<SOFTCAP>(kf0, vf0, kb32 << 5, cpos, window, sc, kb32 == kb_first || kb32 == kb_last, lane);
+      c.template compute<SOFTCAP>(kf0, vf0, kb32 << 5, cpos, window, sc, lane);
       if (kb32 + 1 <= my_last) {
         if (kb32 + 2 <= my_last) fetch(kb32 + 2, kf0, vf0);
-        c.template compute_any<SOFTCAP>(kf1, vf1, (kb32 + 1) << 5, cpos, window, sc, kb32 + 1 == kb_last, lane);
+        c.template compute<SOFTCAP>(kf1, vf1, (kb32 + 1) << 5, cpos, window, sc, lane);
       }
     }
   }
@@ -476,17 +463,13 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
 
 }  // namespace
 
-int g_prefill_variant = 0;     // 0: chosen by the grid's size; 1: whole tiles per wave; 2: keys split over a block's waves
-int g_prefill_heads = 0;       // 0: heads per wave chosen by the grid's size; 1 or 2 force it
-extern "C" void alice_set_prefill_variant(int v, int heads) { g_prefill_variant = v; g_prefill_heads = heads; }
-
 // Head sizes the matrix-core kernels and the fragment cache layout cover.
 extern "C" int alice_attention_mfma_supported(int d) { return d == 64 || d == 128 || d == 256; }
 
 extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
                                        const int* cu_seqlens, const int* context_lens, const int* block_table,
                                        int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
-                                       float scale, float softcap, int window, hipStream_t stream) {
+                                       float scale, float softcap, int window, int variant, hipStream_t stream) {
   ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
   ALICE_CHECK(nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
   ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
@@ -496,8 +479,8 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   const int group = nH / nKV;
   // Two heads a wave halve the key/value reads.
   const long waves2 = (long)ceil_div(max_new, 64) * B * nKV * ceil_div(group, 2) * 4;
-  int gh = group % 2 == 0 ? 2 : 1;
-  if (g_prefill_heads == 1 || (g_prefill_heads == 2 && group % 2 == 0)) gh = g_prefill_heads;
+  const int gh = group % 2 == 0 ? 2 : 1;
+  ALICE_CHECK(variant >= 0 && variant <= 2, "attention: unknown variant %d", variant);
   ALICE_CHECK((long)nKV * ceil_div(group, gh) <= 65535, "attention: too many heads for one launch");
   dim3 grid(ceil_div(max_new, 64), B, nKV * ceil_div(group, gh));
 #define GO(DT, GH)                                                                                                          \
@@ -522,7 +505,7 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   } while (0)
   // Few waves (one prompt of a few thousand tokens): split every tile's keys over four waves.  Many: whole
   // tiles per wave, two heads a wave where the group is even.
-  const bool split = g_prefill_variant == 2 || (g_prefill_variant == 0 && waves2 < 4096);
+  const bool split = variant == ALICE_PREFILL_SPLIT || (variant == ALICE_PREFILL_AUTO && waves2 < 4096);
   if (split) {
     ALICE_CHECK(nH <= 65535, "attention: too many heads for one launch");
     if (d == 64) GOS(2); else if (d == 128) GOS(4); else GOS(8);

@@ -178,97 +178,13 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
   }
 }
 
+constexpr int WM = 8, WN = 4;   // a wave's tile: 8 x 4 MFMA tiles = 128 tokens x 64 output features
+
 // ---------------------------------------------------------------- tiled, many tokens
-// Block: 4 waves side by side along N; every wave computes 128 tokens x 64 output features
-// (8 x 4 MFMA tiles, 128 accumulator registers per lane) and streams its own weight tiles; the four
-// waves read the same activation rows (through the vector cache).  grid.x: groups of 16 row tiles
-// (256 features; for GeGLU 128 output features = 8 gate + 8 up tiles); grid.y: groups of 128 tokens.
-constexpr int WM = 8, WN = 4;
-
-template <int EPI, typename TO, bool FULL>
-__global__ __launch_bounds__(256) void linear_tiled_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
-                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                                float epi) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int m0 = blockIdx.y * (16 * WM);
-  int tile[WN];
-#pragma unroll
-  for (int i = 0; i < WN; ++i) {
-    if (EPI == ALICE_EPI_GEGLU) {
-      const int pair = (blockIdx.x * 4 + wave) * (WN / 2) + (i >> 1);
-      tile[i] = (i & 1) ? N / 16 + pair : pair;
-      if (pair >= N / 16) tile[i] = NT;                    // beyond the matrix
-    } else {
-      tile[i] = (blockIdx.x * 4 + wave) * WN + i;
-    }
-  }
-  int row[WM];
-#pragma unroll
-  for (int j = 0; j < WM; ++j) row[j] = min(m0 + j * 16 + r, M - 1);      // clamped: extra rows are computed and dropped
-
-  f32x4 acc[WN][WM];
-#pragma unroll
-  for (int i = 0; i < WN; ++i)
-#pragma unroll
-    for (int j = 0; j < WM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  u32x4 a[WN], b[WM], an[WN], bn[WM];
-  auto load_tile = [&](int kt, u32x4* aa, u32x4* bb) {
-#pragma unroll
-    for (int i = 0; i < WN; ++i) {
-      aa[i] = u32x4{0u, 0u, 0u, 0u};
-      if (tile[i] < NT) aa[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
-    }
-#pragma unroll
-    for (int j = 0; j < WM; ++j) bb[j] = load_x_frag(x, row[j], true, K, kt, g);
-  };
-  load_tile(0, a, b);
-  for (int kt = 0; kt < KT; ++kt) {
-    if (kt + 1 < KT) load_tile(kt + 1, an, bn);
-#pragma unroll
-    for (int i = 0; i < WN; ++i)
-#pragma unroll
-      for (int j = 0; j < WM; ++j) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
-#pragma unroll
-    for (int i = 0; i < WN; ++i) a[i] = an[i];
-#pragma unroll
-    for (int j = 0; j < WM; ++j) b[j] = bn[j];
-  }
-
-#pragma unroll
-  for (int j = 0; j < WM; ++j) {
-    const int m = m0 + j * 16 + r;
-    if (m >= M) continue;
-    const size_t row_off = (size_t)m * N;
-    if (EPI == ALICE_EPI_GEGLU) {
-#pragma unroll
-      for (int p = 0; p < WN / 2; ++p) {
-        if (tile[2 * p] >= NT) continue;
-        const int n = tile[2 * p] * 16 + g * 4;
-        f32x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
-        store4(y, row_off, n, N, o);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < WN; ++i) {
-        if (tile[i] >= NT) continue;
-        const int n = tile[i] * 16 + g * 4;
-        f32x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
-        store4(y, row_off, n, N, o);
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------- tiled, activations through LDS
-// As above, but the block's 128 tokens x 64 inner elements of activations are staged once in LDS (in
-// fragment order, so LDS reads and writes are linear) and read by all four waves, which cuts the
-// activation traffic from the vector cache by four.  Two stages are kept: while one is used for the
+// Block: 4 waves side by side along N; every wave computes 128 (or 64) tokens x 64 output features
+// (8 x 4 MFMA tiles, 128 accumulator registers per lane) and streams its own weight tiles straight
+// from memory.  The block's tokens x 64 inner elements of activations are staged once in LDS (in
+// fragment order, so LDS reads and writes are linear) and read by all four waves.  Two stages are kept: while one is used for the
 // MFMAs the next one's global loads are in flight, and one barrier per stage suffices.  The grid is
 // one-dimensional and mapped so that the blocks that share weight tiles run on the same XCD (blocks
 // are dealt to the eight XCDs round robin by their linear index).
@@ -407,8 +323,6 @@ __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restr
   dst[o] = (n < N && k < K) ? src[(size_t)n * K + k] : z;
 }
 
-int g_skinny_rt = 0, g_skinny_nw = 0;      // tuning overrides (0: choose by shape)
-
 template <int RT, int MT, int EPI, typename TO>
 int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
@@ -417,8 +331,7 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   dim3 grid(groups, split);
   // Eight waves a block when the slice is long enough to give each of them work and the block count is
   // too low to fill the chip with four.
-  bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
-  if (g_skinny_nw) eight = g_skinny_nw == 8 && RT * MT <= 8;
+  const bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
     linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
@@ -433,7 +346,6 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
 // Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
 // on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)
 int skinny_row_tiles(int M, int N, int epi, int split) {
-  if (g_skinny_rt) return g_skinny_rt;
   const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   if (tiles >= 4096) return 4;
   // Many tokens: more rows per block per read of the activations, wherever the inner dimension can be
@@ -461,14 +373,12 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
   return 1;
 }
 
-int g_tiled_variant = 0;     // 0: activations through LDS; 1: every wave loads its own (for comparison)
-
 template <int EPI, typename TO>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
-  if (g_tiled_variant == 0) {
+  {
     // 128 tokens a block, or 64 when that leaves the chip less than full
     const int per = ceil_div(KT, split);
     if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
@@ -479,9 +389,6 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
       linear_tiled_lds_kernel<EPI, TO, false, 4><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
     }
-  } else {
-    dim3 grid(gx, gy);
-    linear_tiled_mfma_kernel<EPI, TO, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi);
   }
   ALICE_LAUNCH_CHECK();
   return 0;
@@ -490,8 +397,6 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
 }  // namespace
 
 extern "C" int alice_has_mfma_linear() { return 1; }
-extern "C" void alice_set_tiled_variant(int v) { g_tiled_variant = v; }
-extern "C" void alice_set_skinny_override(int row_tiles, int waves) { g_skinny_rt = row_tiles; g_skinny_nw = waves; }
 
 // Whether a matrix of `rows` x K with this epilogue can use the fragment layout.
 extern "C" int alice_frag16_supported(int rows, int K, int epilogue) {
@@ -515,7 +420,7 @@ int alice_linear_split_hint_frag(int M, int N, int K) {
     // or quarter the inner dimension instead of the tile.
     const int blocks = ceil_div(N, 256) * ceil_div(M, 128), KT = (K + 31) / 32;
     if (blocks >= 200 || KT < 32) return 1;
-    return (blocks < 200 && KT >= 256) ? 4 : 2;
+    return 2;
   }
   const int KT = (K + 31) / 32;
   if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);
@@ -539,7 +444,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   // blocks for the tiled kernel, which shares the activations through LDS, as soon as there are 17 tokens.
   bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 16 && N >= 65536 && split_k == 1));
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
-  ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && (skinny || g_tiled_variant == 0)),
+  ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),
               "linear: partial sums need no epilogue and float32 output");
   ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
 #define BY_EPI(FN, ...)                                                                            \

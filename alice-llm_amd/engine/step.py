@@ -58,6 +58,32 @@ def _bucket(n: int) -> int:
 CONTEXT_BUCKET = 512        # captured decode steps are specialised to the context length rounded up to this
 
 
+class _Staging:
+    """Pinned host buffers for the small integer arrays of a step, reused in turn; a buffer is written again
+    only after the copy that last read it has run (pinned memory is allocated once, not per step)."""
+
+    def __init__(self, n_buffers: int = 4):
+        self.buffers = [None] * n_buffers
+        self.events = [None] * n_buffers
+        self.turn = 0
+
+    def upload(self, values: List[int], device) -> torch.Tensor:
+        i = self.turn = (self.turn + 1) % len(self.buffers)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        n = len(values)
+        if self.buffers[i] is None or self.buffers[i].numel() < n:
+            self.buffers[i] = torch.empty(max(1024, 2 * n), dtype=torch.int32).pin_memory()
+        host = self.buffers[i][:n]
+        host.copy_(torch.tensor(values, dtype=torch.int32))
+        out = torch.empty(n, dtype=torch.int32, device=device)
+        out.copy_(host, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+        return out
+
+
 class _DecodeGraph:
     """One captured decode step: its static integer inputs, its static logits, and pinned staging buffers."""
 
@@ -138,6 +164,7 @@ class Engine:
         self.use_graphs = safe if use_graphs is None else (use_graphs and safe)
         self._graphs = {}
         self._max_graphs = max_graphs
+        self._staging = _Staging()
 
     # ------------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> List[int]:
@@ -202,7 +229,7 @@ class Engine:
 
         # one host-to-device copy for all the small integer arrays of the step
         pieces = [flat, positions, seq_of, list(slots), rows, cu, ctx_lens] + [sum(t, []) for t in tables]
-        packed = torch.tensor(sum(pieces, []), dtype=torch.int32).pin_memory().to(self.device, non_blocking=True)
+        packed = self._staging.upload(sum(pieces, []), self.device)
         offs = [0]
         for p in pieces:
             offs.append(offs[-1] + len(p))

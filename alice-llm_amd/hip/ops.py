@@ -44,7 +44,7 @@ def _declare(lib) -> None:
         "alice_frag16_supported": [I, I, I],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
-        "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
+        "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -325,8 +325,14 @@ def decode_splits(n_seqs: int, num_kv_heads: int, max_context: int) -> int:
     return max(1, min(by_fill, by_work, 64))
 
 
+PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT = 0, 1, 2
+
+
 def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_table, *, num_heads: int, n_seqs: int,
-                      max_new: int, max_context: int, scale: float, softcap: Optional[float], window: Optional[int]) -> None:
+                      max_new: int, max_context: int, scale: float, softcap: Optional[float], window: Optional[int],
+                      variant: int = PREFILL_AUTO) -> None:
+    """Prompt attention on the matrix cores.  variant: whole query tiles per wave, or one tile's keys split over
+    a block's four waves (what fills the chip when there are few tiles); AUTO picks by the grid's size."""
     n_pages, nKV, page_size, d = k_pool.shape
     T = q.shape[0]
     _dev(q, "q", torch.bfloat16, (T, num_heads * d))
@@ -340,7 +346,8 @@ def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_ta
         raise HipLibraryError(f"{max_context} keys are beyond the block table {tuple(block_table.shape)}")
     _call("alice_attention_prefill", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
           cu_seqlens.data_ptr(), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_seqs,
-          max_new, num_heads, nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), _stream())
+          max_new, num_heads, nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), int(variant),
+          _stream())
 
 
 def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,

@@ -446,10 +446,11 @@ def test_fragment_cache_layout_is_what_the_comment_says():
 def test_attention_mfma_prompts(nH, nKV, d, cap, window):
     for lens, new in (((5, 130, 66), (5, 130, 66)), ((150, 64, 33), (20, 3, 33)), ((300,), (300,))):
         q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, new, cap, window, seed=3)
-        out = torch.full_like(q, float("nan"))
-        ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
-                              max_context=max(lens), scale=scale, softcap=cap, window=window)
-        close(out, ref, 2e-2)
+        for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_AUTO):
+            out = torch.full_like(q, float("nan"))
+            ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
+                                  max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant)
+            close(out, ref, 2e-2)
 
 
 @pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
@@ -462,11 +463,12 @@ def test_attention_mfma_single_tokens(nH, nKV, d, cap, window):
         ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=cap,
                              window=window, splits=splits)
         close(out, ref, 2e-2)
-    # the prompt kernel on single tokens gives the same
-    out = torch.full_like(q, float("nan"))
-    ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=1, max_context=max(lens),
-                          scale=scale, softcap=cap, window=window)
-    close(out, ref, 2e-2)
+    # the prompt kernels on single tokens give the same
+    for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT):
+        out = torch.full_like(q, float("nan"))
+        ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=1, max_context=max(lens),
+                              scale=scale, softcap=cap, window=window, variant=variant)
+        close(out, ref, 2e-2)
 
 
 def test_attention_mfma_far_key_and_window_edge():
@@ -475,13 +477,13 @@ def test_attention_mfma_far_key_and_window_edge():
         k[3] = 0; k[3, :, 0] = 40.0
         q[L - 1] = 0; q[L - 1, :, 0] = 40.0
     q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, None, seed=5, crafted=far)
-    for fn in ("decode", "prefill"):
+    for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT):
         out = torch.full_like(q, float("nan"))
         if fn == "decode":
             ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=None)
         else:
             ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=1, max_new=1, max_context=L, scale=scale,
-                                  softcap=None, window=None)
+                                  softcap=None, window=None, variant=fn)
         close(out, ref, 2e-2)
         assert (out.view(nH, d)[0].double().cpu() - ref.view(nH, d)[0]).abs().max() < 2e-2 and ref.view(nH, d)[0].abs().max() > 0.1
     for where, seen in ((L - 101, False), (L - 100, True)):
@@ -489,13 +491,13 @@ def test_attention_mfma_far_key_and_window_edge():
             k[where] = 0; k[where, :, 0] = 40.0; v[where] = 7.0
             q[L - 1] = 0; q[L - 1, :, 0] = 40.0
         q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, 100, seed=6, crafted=edge)
-        for fn in ("decode", "prefill"):
+        for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT):
             out = torch.full_like(q, float("nan"))
             if fn == "decode":
                 ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=100)
             else:
                 ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=1, max_new=1, max_context=L,
-                                      scale=scale, softcap=None, window=100)
+                                      scale=scale, softcap=None, window=100, variant=fn)
             close(out, ref, 2e-2)
             assert (abs(float(out[0, 0]) - 7.0) < 5e-2) == seen
 
