@@ -36,16 +36,18 @@ int alice_embed(const int* tokens, const void* table, int table_dtype, int table
 int alice_add_norm(float* resid, const float* branch, int n_partials, long partial_stride,
                    const void* w_post, const void* w_pre, int w_dtype, void* out, int out_dtype,
                    const int* rows, int T, int H, float eps_post, float eps_pre, float off_post,
-                   float off_pre, int full_precision, hipStream_t stream);
+                   float off_pre, int full_precision, int out_layout, hipStream_t stream);
 
 int alice_softcap(float* x, long n, float cap, int full_precision, hipStream_t stream);
 
 // y[M, N] = x[M, K] . W^T with an optional epilogue.  `variant` forces a kernel (tests); AUTO picks.
 // For GEGLU, W has 2N rows.  `split_k` > 1 asks for partial sums y[split_k][M][N] in float32
 // (no epilogue), to be added up by the consumer (alice_add_norm's n_partials).
+// x_layout / y_layout: ALICE_LAYOUT_ROW, or ALICE_LAYOUT_FRAG16 for activations stored in fragment order
+// ([M/16][K/32][64][8], bfloat16, rows padded to 16), which the producers of a decode step write.
 int alice_linear(const void* x, int x_dtype, const void* w, int w_dtype, int w_layout, void* y, int y_dtype,
                  int M, int N, int K, int epilogue, float epi_param, int split_k, int variant,
-                 int full_precision, hipStream_t stream);
+                 int full_precision, int x_layout, int y_layout, hipStream_t stream);
 // How many partial sums AUTO would like for this shape (1 = none).
 int alice_linear_split_hint(int M, int N, int K, int w_layout);
 
@@ -77,7 +79,7 @@ long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                            const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
                            int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
-                           hipStream_t stream);
+                           int out_layout, hipStream_t stream);
 
 // Lowest index among equal maxima.
 int alice_argmax_chunks(int B, int V);

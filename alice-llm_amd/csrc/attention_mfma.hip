@@ -353,6 +353,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
   }
 }
 
+// Where output element (sequence b, column c of nH * D) goes: row-major, or fragment order for the output
+// projection's streaming kernel ([B/16][nH*D/32][64][8]).
+__device__ __forceinline__ size_t decode_out_index(int layout, int b, int c, int width) {
+  if (layout == 0) return (size_t)b * width + c;
+  return ((size_t)((size_t)(b >> 4) * (width >> 5) + (c >> 5)) * 64 + ((c & 31) >> 3) * 16 + (b & 15)) * 8 + (c & 7);
+}
+
 // ---------------------------------------------------------------- single tokens, keys split over blocks
 // grid: (sequences, kv heads, splits).  The query tile's 16 columns are the query heads of the kv head's
 // group (group <= 16).  The sequence's 32-key blocks are dealt out in contiguous runs to the
@@ -363,7 +370,8 @@ template <int DT, bool SOFTCAP>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, float* __restrict__ parts, const int* __restrict__ context_lens,
-    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int splits) {
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int splits,
+    int out_layout) {
   constexpr int D = DT * 32;
   __shared__ float sm[4][16], sl[4][16];
   extern __shared__ __align__(16) float so[];            // [4 waves][group][D + 4]
@@ -435,7 +443,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
     const int head = kvh * group + hc;
     if (splits == 1) {
-      out[((size_t)b * nH + head) * D + e] = f32_to_bf16(acc / ll);
+      out[decode_out_index(out_layout, b, head * D + e, nH * D)] = f32_to_bf16(acc / ll);
     } else {
       float* pr = parts + (((size_t)b * nH + head) * splits + split) * (D + 2);
       pr[2 + e] = acc;
@@ -445,7 +453,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 // Combines the splits of one (sequence, head) in the order 0, 1, ...: grid (sequences * heads), D threads.
-__global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits) {
+__global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits,
+                                          int nH, int out_layout) {
   const float* pr = parts + (size_t)blockIdx.x * splits * (D + 2);
   float mm = -INFINITY;
   for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[(size_t)s * (D + 2)]);
@@ -457,7 +466,7 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
       acc += ps[2 + e] * f;
       ll += ps[1] * f;
     }
-    out[(size_t)blockIdx.x * D + e] = f32_to_bf16(acc / ll);
+    out[decode_out_index(out_layout, blockIdx.x / nH, (blockIdx.x % nH) * D + e, nH * D)] = f32_to_bf16(acc / ll);
   }
 }
 
@@ -528,13 +537,14 @@ extern "C" long alice_attention_decode_workspace(int B, int nH, int d, int split
 extern "C" int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                                       const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
                                       int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
-                                      hipStream_t stream) {
+                                      int out_layout, hipStream_t stream) {
   ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
   ALICE_CHECK(nKV >= 1 && nH % nKV == 0 && nH / nKV <= 16, "attention (decode): %d query heads per kv head are more than the 16 this kernel takes", nKV ? nH / nKV : 0);
   ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
   ALICE_CHECK(B >= 0 && nKV <= 65535 && splits >= 1 && splits <= 64, "attention: bad batch B=%d or splits=%d", B, splits);
   ALICE_CHECK(splits == 1 || parts != nullptr, "attention: split keys need the workspace");
   ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
+  ALICE_CHECK(out_layout == 0 || out_layout == 1, "attention: unknown output layout %d", out_layout);
   if (B == 0) return 0;
   dim3 grid(B, nKV, splits);
   const size_t lds = (size_t)4 * (nH / nKV) * (d + 4) * sizeof(float);
@@ -542,16 +552,16 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
   do {                                                                                                                      \
     if (softcap > 0.f)                                                                                                      \
       attn_decode_kernel<DT, true><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits);              \
+          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits, out_layout);  \
     else                                                                                                                    \
       attn_decode_kernel<DT, false><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits);              \
+          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits, out_layout);  \
   } while (0)
   if (d == 64) GO(2); else if (d == 128) GO(4); else GO(8);
 #undef GO
   ALICE_LAUNCH_CHECK();
   if (splits > 1) {
-    attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits);
+    attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits, nH, out_layout);
     ALICE_LAUNCH_CHECK();
   }
   return 0;

@@ -51,6 +51,13 @@ extern "C" int alice_embed(const int* tokens, const void* table, int table_dtype
   return 0;
 }
 
+// Where element (row r, column i) of a [T, H] bfloat16 output goes: row-major, or fragment order for the
+// matrix-core kernels ([T/16][H/32][64][8], see linear_mfma.hip).
+__device__ __forceinline__ size_t out_index(int layout, int r, int i, int H) {
+  if (layout == 0) return (size_t)r * H + i;
+  return ((size_t)((size_t)(r >> 4) * (H >> 5) + (i >> 5)) * 64 + ((i & 31) >> 3) * 16 + (r & 15)) * 8 + (i & 7);
+}
+
 // ---------------------------------------------------------------- residual add + norms
 // One block per row r (source row rows ? rows[r] : r):
 //   b   = sum over `n_partials` slices of `branch` (slice stride `partial_stride` elements)
@@ -64,7 +71,7 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const float* __restri
                                 int n_partials, size_t partial_stride,
                                 const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
                                 TO* __restrict__ out, const int* __restrict__ rows, int H,
-                                float eps_post, float eps_pre, float off_post, float off_pre) {
+                                float eps_post, float eps_pre, float off_post, float off_pre, int out_layout) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t src = (size_t)(rows ? rows[r] : r) * H;
@@ -99,9 +106,9 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const float* __restri
     }
   }
   if (!out) return;
-  TO* o = out + (size_t)r * H;
+  TO* o = out;
   if (!w_pre) {
-    for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(o, i, x[i]);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(o, out_index(out_layout, r, i, H), x[i]);
     return;
   }
   ss_x = block_sum(ss_x, red);
@@ -109,7 +116,7 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const float* __restri
   float inv = FULL ? 1.f / sqrtf(mean + eps_pre) : rsqrtf(mean + eps_pre);
   // Each thread re-reads the elements it wrote itself above, so no barrier is needed.
   for (int i = threadIdx.x; i < H; i += blockDim.x)
-    store_f32(o, i, x[i] * inv * (off_pre + load_f32(w_pre, i)));
+    store_f32(o, out_index(out_layout, r, i, H), x[i] * inv * (off_pre + load_f32(w_pre, i)));
 }
 
 // The same operation with a row held in registers (EPT elements per thread): every operand is read
@@ -119,7 +126,7 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
                                      int n_partials, size_t partial_stride,
                                      const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
                                      TO* __restrict__ out, const int* __restrict__ rows, int H,
-                                     float eps_post, float eps_pre, float off_post, float off_pre) {
+                                     float eps_post, float eps_pre, float off_post, float off_pre, int out_layout) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t src = (size_t)(rows ? rows[r] : r) * H;
@@ -168,7 +175,7 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
     }
   }
   if (!out) return;
-  TO* o = out + (size_t)r * H;
+  TO* o = out;
   float inv = 1.f;
   if (w_pre) {
     float ss = 0.f;
@@ -181,19 +188,21 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int i = threadIdx.x + j * blockDim.x;
-    if (i < H) store_f32(o, i, w_pre ? xv[j] * inv * (off_pre + wq[j]) : xv[j]);
+    if (i < H) store_f32(o, out_index(out_layout, r, i, H), w_pre ? xv[j] * inv * (off_pre + wq[j]) : xv[j]);
   }
 }
 
 extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials, long partial_stride,
                               const void* w_post, const void* w_pre, int w_dtype, void* out, int out_dtype,
                               const int* rows, int T, int H, float eps_post, float eps_pre,
-                              float off_post, float off_pre, int full_precision, hipStream_t stream) {
+                              float off_post, float off_pre, int full_precision, int out_layout, hipStream_t stream) {
   ALICE_CHECK(T >= 0 && H > 0, "add_norm: bad sizes T=%d H=%d", T, H);
   ALICE_CHECK(resid != nullptr, "add_norm: the residual stream is missing");
   ALICE_CHECK(dtype_ok(w_dtype) && dtype_ok(out_dtype), "add_norm: unknown dtype");
   ALICE_CHECK(!(rows && branch), "add_norm: a row gather cannot be combined with a residual add");
   ALICE_CHECK(n_partials >= 1 && n_partials <= 64, "add_norm: n_partials %d out of range", n_partials);
+  ALICE_CHECK(out_layout == 0 || (out_layout == 1 && out && out_dtype == DT_BF16 && H % 32 == 0),
+              "add_norm: output in fragment order needs bfloat16 and a width that is a multiple of 32");
   if (T == 0) return 0;
   // Rows up to 8192 wide are held in registers: 256 threads x 1..4 elements, then 1024 threads x 4 or 8.
   int threads = H >= 2048 ? 512 : 256, ept = 0;
@@ -201,7 +210,7 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
   else if (H <= 4096) { threads = 1024; ept = 4; }
   else if (H <= 8192) { threads = 1024; ept = 8; }
 #define ARGS resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, \
-             eps_post, eps_pre, off_post, off_pre
+             eps_post, eps_pre, off_post, off_pre, out_layout
 #define LAUNCH(TW, TO, FULL)                                                                         \
   do {                                                                                               \
     if (ept == 1) add_norm_regs_kernel<TW, TO, FULL, 1><<<T, threads, 0, stream>>>(ARGS);            \

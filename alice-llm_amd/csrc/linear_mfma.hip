@@ -38,6 +38,14 @@ __device__ __forceinline__ u32x4 load_x_frag(const bf16_t* __restrict__ x, int r
   return v;
 }
 
+// The same fragment when the activations themselves are stored in fragment order
+// ([M/16][K/32][64 lanes][8], what a decode step's producers write): one contiguous 1 KB read per wave.
+__device__ __forceinline__ u32x4 load_x_frag_f(const bf16_t* __restrict__ x, int mtile, bool ok, int KT, int kt, int lane) {
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (ok) v = *reinterpret_cast<const u32x4*>(x + ((size_t)((size_t)mtile * KT + kt) * 64 + lane) * 8);
+  return v;
+}
+
 template <int EPI, bool FULL>
 __device__ __forceinline__ float epilogue1(float v, float p) {
   if (EPI == ALICE_EPI_SOFTCAP) return p * (FULL ? tanh_full(v / p) : tanh_fast(v / p));
@@ -62,6 +70,15 @@ __device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n
   }
 }
 
+// Four consecutive output features of token m, stored in fragment order for the next matrix product
+// (its inner dimension is this one's N): element (m, n) lies at
+// ((m/16 * N/32 + n/32) * 64 + (n%32)/8 * 16 + m%16) * 8 + n%8.  N is a multiple of 32, n of 4.
+__device__ __forceinline__ void store4_frag(bf16_t* __restrict__ y, int m, int n, int N, f32x4 v) {
+  const size_t off = ((size_t)((size_t)(m >> 4) * (N >> 5) + (n >> 5)) * 64 + ((n & 31) >> 3) * 16 + (m & 15)) * 8 + (n & 7);
+  uint2 pk = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+  *reinterpret_cast<uint2*>(y + off) = pk;
+}
+
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
 // Block: NW waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + NW, ...; the parts of
 // waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
@@ -70,7 +87,7 @@ __device__ __forceinline__ void store4(TO* __restrict__ y, size_t row_off, int n
 template <int RT, int MT, int NW, int EPI, typename TO, bool FULL>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                            int kt_per_slice, float epi) {
+                                                            int kt_per_slice, float epi, int x_frag, int y_frag) {
   extern __shared__ __align__(16) float red[];            // [NW - 1][RT*MT][64][4]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -108,7 +125,8 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
         aa[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
     }
 #pragma unroll
-    for (int j = 0; j < MT; ++j) bb[j] = load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
+    for (int j = 0; j < MT; ++j)
+      bb[j] = x_frag ? load_x_frag_f(x, j, kok, KT, kt, lane) : load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
   };
   // Blocks start at different places of their k range and wrap around: all blocks read the same
   // activations, and in lockstep they would all ask the same L2 channel for the same line at once.
@@ -163,6 +181,9 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
         f32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = gelu_tanh_f(acc[2 * p][j][i], FULL) * acc[2 * p + 1][j][i];
+        if constexpr (sizeof(TO) == 2) {
+          if (y_frag) { if (n < N) store4_frag((bf16_t*)yo, row[j], n, N, o); continue; }
+        }
         store4(yo, row_off, n, N, o);
       }
     } else {
@@ -172,6 +193,9 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
         f32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
+        if constexpr (sizeof(TO) == 2) {
+          if (y_frag) { if (n < N) store4_frag((bf16_t*)yo, row[j], n, N, o); continue; }
+        }
         store4(yo, row_off, n, N, o);
       }
     }
@@ -190,7 +214,9 @@ constexpr int WM = 8, WN = 4;   // a wave's tile: 8 x 4 MFMA tiles = 128 tokens 
 // are dealt to the eight XCDs round robin by their linear index).
 constexpr int KC = 2;      // k-tiles per stage
 
-template <int EPI, typename TO, bool FULL, int TM>
+// XF: the activations come in fragment order (a compile-time choice: as a run-time one it cost the
+// row-major path a third of its speed).
+template <int EPI, typename TO, bool FULL, int TM, bool XF>
 __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
                                                                float epi, int gx, int gy, int kt_per_slice) {
@@ -234,7 +260,11 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
 #pragma unroll
     for (int kc = 0; kc < KC; ++kc)
 #pragma unroll
-      for (int j = 0; j < XJ; ++j) xr[kc][j] = load_x_frag(x, xrow[j], kt_base + s * KC + kc < kt_end, K, kt_base + s * KC + kc, g);
+      for (int j = 0; j < XJ; ++j) {
+        const int kt = kt_base + s * KC + kc;
+        if constexpr (XF) xr[kc][j] = load_x_frag_f(x, min((m0 >> 4) + XJ * wave + j, (M - 1) >> 4), kt < kt_end, KT, kt, lane);
+        else xr[kc][j] = load_x_frag(x, xrow[j], kt < kt_end, K, kt, g);
+      }
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
@@ -324,7 +354,8 @@ __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restr
 }
 
 template <int RT, int MT, int EPI, typename TO>
-int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
+int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
+                  hipStream_t s) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int groups = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, RT / 2) : ceil_div(NT, RT);
   const int per = ceil_div(KT, split);
@@ -334,10 +365,10 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   const bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
-    linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+    linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, x_frag, y_frag);
   } else {
     const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-    linear_skinny_kernel<RT, MT, 4, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi);
+    linear_skinny_kernel<RT, MT, 4, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, x_frag, y_frag);
   }
   ALICE_LAUNCH_CHECK();
   return 0;
@@ -356,9 +387,10 @@ int skinny_row_tiles(int M, int N, int epi, int split) {
 }
 
 template <int EPI, typename TO>
-int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
+int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
+                    hipStream_t s) {
   const int rt = skinny_row_tiles(M, N, EPI, split);
-#define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, s)
+#define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, x_frag, y_frag, s)
 #define BY_RT(MT)                                                   \
   do {                                                              \
     if (rt == 4) GO(4, MT);                                         \
@@ -374,20 +406,26 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
 }
 
 template <int EPI, typename TO>
-int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, hipStream_t s) {
+int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
+                 hipStream_t s) {
+  (void)y_frag;
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
   {
     // 128 tokens a block, or 64 when that leaves the chip less than full
     const int per = ceil_div(KT, split);
-    if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
+    if (x_frag) {
+      // fragment order is what decode steps use: few tokens, one or a few block rows
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 8><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+      linear_tiled_lds_kernel<EPI, TO, false, 8, true><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+    } else if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
+      dim3 grid(8 * ceil_div(gx * gy, 8), split);
+      linear_tiled_lds_kernel<EPI, TO, false, 8, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
     } else {
       gy = ceil_div(M, 64);
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 4><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+      linear_tiled_lds_kernel<EPI, TO, false, 4, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
     }
   }
   ALICE_LAUNCH_CHECK();
@@ -432,13 +470,16 @@ int alice_linear_split_hint_frag(int M, int N, int K) {
 }
 
 int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_dtype, int M, int N, int K,
-                      int epi, float epi_param, int split_k, int variant, hipStream_t stream) {
+                      int epi, float epi_param, int split_k, int variant, int x_layout, int y_layout,
+                      hipStream_t stream) {
   ALICE_CHECK(x_dtype == DT_BF16, "linear: the fragment layout needs bfloat16 activations");
   ALICE_CHECK(dtype_ok(y_dtype), "linear: unknown output dtype");
   ALICE_CHECK(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear: bad sizes M=%d N=%d K=%d (K must be a multiple of 8)", M, N, K);
   ALICE_CHECK(epi != ALICE_EPI_GEGLU || N % 16 == 0, "linear: GeGLU in the fragment layout needs N %% 16 == 0, found %d", N);
   ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f, "linear: softcap must be positive");
   ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0, "linear: operands must be 16-byte aligned");
+  ALICE_CHECK(x_layout == ALICE_LAYOUT_ROW || (x_layout == ALICE_LAYOUT_FRAG16 && K % 32 == 0),
+              "linear: activations in fragment order need K %% 32 == 0, found K=%d", K);
   if (M == 0) return 0;
   // Up to 64 tokens stream the weights once; very wide matrices (the output head) have enough column
   // blocks for the tiled kernel, which shares the activations through LDS, as soon as there are 17 tokens.
@@ -447,6 +488,10 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),
               "linear: partial sums need no epilogue and float32 output");
   ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
+  ALICE_CHECK(y_layout == ALICE_LAYOUT_ROW || (y_layout == ALICE_LAYOUT_FRAG16 && skinny && y_dtype == DT_BF16 && N % 32 == 0 &&
+                                                split_k == 1 && epi != ALICE_EPI_SOFTCAP),
+              "linear: output in fragment order needs the streaming kernel, bfloat16 and N %% 32 == 0");
+  const int x_frag = x_layout == ALICE_LAYOUT_FRAG16, y_frag = y_layout == ALICE_LAYOUT_FRAG16;
 #define BY_EPI(FN, ...)                                                                            \
   do {                                                                                             \
     if (y_dtype == DT_F32) {                                                                       \
@@ -459,7 +504,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
       return FN<ALICE_EPI_SOFTCAP, bf16_t>(__VA_ARGS__);                                           \
     }                                                                                              \
   } while (0)
-  if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, stream);
-  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, stream);
+  if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
+  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
 #undef BY_EPI
 }

@@ -131,5 +131,6 @@ class CausalLM:
         if ctx.want_rows is None or ctx.want_rows.numel() == 0:
             stream.flush()
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
-        normed = stream.rows_normed(self.final_norm, ctx.want_rows)
+        frag = getattr(ctx, "fragment_activations", False) and getattr(self.head, "accepts_fragment_activations", False)
+        normed = stream.rows_normed(self.final_norm, ctx.want_rows, fragments=frag)
         return self.head.forward(normed)

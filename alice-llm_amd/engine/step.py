@@ -40,6 +40,9 @@ class StepContext:
     new_lens: Sequence[int] = ()
     start_lens: Sequence[int] = ()
     slot_ids: Sequence[int] = ()
+    # decode steps of at most 64 sequences in bfloat16: activations between the built-in parts travel in the
+    # matrix-core kernels' fragment order (parts that do not declare support get plain tensors)
+    fragment_activations: bool = False
 
 
 Want = Union[str, Sequence[Sequence[int]]]
@@ -106,7 +109,8 @@ class _DecodeGraph:
         self.ctx = StepContext(tokens=part(0), positions=part(1), seq_of_token=part(2), slots=part(3), want_rows=part(4),
                                cu_seqlens=part(5), context_lens=part(6), n_tokens=B, n_seqs=B, is_decode=True,
                                max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
-                               start_lens=[0] * B, slot_ids=[0] * B)
+                               start_lens=[0] * B, slot_ids=[0] * B,
+                               fragment_activations=engine.model.precision.act == torch.bfloat16 and B <= 64)
         self.graph = None
         self.logits = None
         self.tables_version = None
@@ -239,7 +243,9 @@ class Engine:
                           want_rows=part(4) if rows else None, cu_seqlens=part(5), context_lens=part(6),
                           n_tokens=T, n_seqs=B, is_decode=all(n == 1 for n in n_new), max_new=max(n_new),
                           max_context=max(ctx_lens), max_position=max(ctx_lens) - 1,
-                          new_lens=n_new, start_lens=start, slot_ids=list(slots))
+                          new_lens=n_new, start_lens=start, slot_ids=list(slots),
+                          fragment_activations=(self.model.precision.act == torch.bfloat16 and T <= 64
+                                                and all(n == 1 for n in n_new)))
         logits = self.model.forward(ctx, self.cache, block_tables)
         self.cache.commit(slots, n_new)
         return logits

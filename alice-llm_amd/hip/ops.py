@@ -36,16 +36,16 @@ def _declare(lib) -> None:
     lib.alice_device_arch.argtypes = [c.c_char_p, I]
     sigs = {
         "alice_embed": [P, P, I, I, P, I, I, I, F, P],
-        "alice_add_norm": [P, P, I, L, P, P, I, P, I, P, I, I, F, F, F, F, I, P],
+        "alice_add_norm": [P, P, I, L, P, P, I, P, I, P, I, I, F, F, F, F, I, I, P],
         "alice_softcap": [P, L, F, I, P],
-        "alice_linear": [P, I, P, I, I, P, I, I, I, I, I, F, I, I, I, P],
+        "alice_linear": [P, I, P, I, I, P, I, I, I, I, I, F, I, I, I, I, I, P],
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
         "alice_frag16_supported": [I, I, I],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
-        "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
+        "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
         "alice_argmax_chunks": [I, I],
@@ -156,8 +156,10 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: f
 def add_norm(resid: torch.Tensor, branch: Optional[torch.Tensor], w_post: Optional[torch.Tensor],
              w_pre: Optional[torch.Tensor], out: Optional[torch.Tensor], *, eps_post: float = 0.0,
              eps_pre: float = 0.0, off_post: float = 0.0, off_pre: float = 0.0,
-             rows: Optional[torch.Tensor] = None, n_partials: int = 1, full_precision: bool) -> None:
-    """resid += norm_post(sum of branch partials); out = norm_pre(resid).  Each piece is optional."""
+             rows: Optional[torch.Tensor] = None, n_partials: int = 1, full_precision: bool,
+             out_layout: int = LAYOUT_ROW) -> None:
+    """resid += norm_post(sum of branch partials); out = norm_pre(resid).  Each piece is optional.
+    out_layout FRAG16: `out` is a flat bfloat16 buffer of ceil16(T) * H elements in fragment order."""
     if resid.dim() != 2:
         raise HipLibraryError("resid must be [T, H]")
     Tres, H = resid.shape
@@ -179,7 +181,9 @@ def add_norm(resid: torch.Tensor, branch: Optional[torch.Tensor], w_post: Option
             w_dtype = w.dtype
     if w_post is not None and branch is None:
         raise HipLibraryError("w_post without a branch")
-    if out is not None:
+    if out is not None and out_layout == LAYOUT_FRAG16:
+        _dev(out, "out", torch.bfloat16, (frag_rows(T) * H,))
+    elif out is not None:
         _dev(out, "out", None, (T, H))
     elif w_pre is not None:
         raise HipLibraryError("w_pre without an output")
@@ -189,7 +193,12 @@ def add_norm(resid: torch.Tensor, branch: Optional[torch.Tensor], w_post: Option
           _opt(w_post, "w_post"), _opt(w_pre, "w_pre"), dtype_code(w_dtype or torch.float32),
           _opt(out, "out"), dtype_code(out.dtype if out is not None else torch.float32),
           _opt(rows, "rows"), T, H, float(eps_post), float(eps_pre), float(off_post), float(off_pre),
-          int(full_precision), _stream())
+          int(full_precision), int(out_layout), _stream())
+
+
+def frag_rows(rows: int) -> int:
+    """Rows of an activation buffer in fragment order: padded to whole tiles of 16."""
+    return -(-rows // 16) * 16
 
 
 def softcap_(x: torch.Tensor, cap: float, full_precision: bool) -> None:
@@ -199,12 +208,21 @@ def softcap_(x: torch.Tensor, cap: float, full_precision: bool) -> None:
 
 def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, n_out: int, k_in: int,
            layout: int = LAYOUT_ROW, epilogue: int = EPI_NONE, epi_param: float = 0.0,
-           split_k: int = 1, variant: int = LINEAR_AUTO, full_precision: bool) -> None:
-    """y = x . W^T.  W: [n_out (2 n_out for GeGLU), k_in] row-major, or its fragment layout."""
-    if x.dim() != 2 or x.shape[1] != k_in:
-        raise HipLibraryError(f"x must be [M, {k_in}], found {tuple(x.shape)}")
-    M = x.shape[0]
-    _dev(x, "x")
+           split_k: int = 1, variant: int = LINEAR_AUTO, full_precision: bool, rows: Optional[int] = None,
+           x_layout: int = LAYOUT_ROW, y_layout: int = LAYOUT_ROW) -> None:
+    """y = x . W^T.  W: [n_out (2 n_out for GeGLU), k_in] row-major, or its fragment layout.
+    x_layout / y_layout FRAG16: activations as flat bfloat16 buffers of ceil16(rows) * width elements in
+    fragment order (then `rows` gives M)."""
+    if x_layout == LAYOUT_FRAG16:
+        if rows is None:
+            raise HipLibraryError("activations in fragment order need the number of rows")
+        M = rows
+        _dev(x, "x", torch.bfloat16, (frag_rows(M) * k_in,))
+    else:
+        if x.dim() != 2 or x.shape[1] != k_in:
+            raise HipLibraryError(f"x must be [M, {k_in}], found {tuple(x.shape)}")
+        M = x.shape[0]
+        _dev(x, "x")
     w_rows = n_out * (2 if epilogue == EPI_GEGLU else 1)
     if layout == LAYOUT_ROW:
         _dev(w, "w", None, (w_rows, k_in))
@@ -213,13 +231,16 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, n_out: int, k_i
         need = ((w_rows + 15) // 16 * 16) * ((k_in + 31) // 32 * 32)
         if w.numel() != need:
             raise HipLibraryError(f"w in fragment layout must hold {need} elements, found {w.numel()}")
-    want = (split_k, M, n_out) if split_k > 1 else (M, n_out)
-    _dev(y, "y", None, want)
+    if y_layout == LAYOUT_FRAG16:
+        _dev(y, "y", torch.bfloat16, (frag_rows(M) * n_out,))
+    else:
+        want = (split_k, M, n_out) if split_k > 1 else (M, n_out)
+        _dev(y, "y", None, want)
     if split_k > 1 and y.dtype != torch.float32:
         raise HipLibraryError("partial sums are float32")
     _call("alice_linear", x.data_ptr(), dtype_code(x.dtype), w.data_ptr(), dtype_code(w.dtype), layout,
           y.data_ptr(), dtype_code(y.dtype), M, n_out, k_in, epilogue, float(epi_param), split_k, variant,
-          int(full_precision), _stream())
+          int(full_precision), int(x_layout), int(y_layout), _stream())
 
 
 def linear_split_hint(M: int, N: int, K: int, layout: int) -> int:
@@ -351,11 +372,16 @@ def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_ta
 
 
 def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,
-                     scale: float, softcap: Optional[float], window: Optional[int], splits: Optional[int] = None) -> None:
+                     scale: float, softcap: Optional[float], window: Optional[int], splits: Optional[int] = None,
+                     out_layout: int = LAYOUT_ROW) -> None:
+    """out_layout FRAG16: `out` is a flat buffer of ceil16(B) * num_heads * d elements in fragment order."""
     n_pages, nKV, page_size, d = k_pool.shape
     B = q.shape[0]
     _dev(q, "q", torch.bfloat16, (B, num_heads * d))
-    _dev(out, "out", torch.bfloat16, (B, num_heads * d))
+    if out_layout == LAYOUT_FRAG16:
+        _dev(out, "out", torch.bfloat16, (frag_rows(B) * num_heads * d,))
+    else:
+        _dev(out, "out", torch.bfloat16, (B, num_heads * d))
     _dev(k_pool, "k_pool", torch.bfloat16)
     _dev(v_pool, "v_pool", torch.bfloat16, k_pool.shape)
     _dev(context_lens, "context_lens", torch.int32, (B,))
@@ -368,25 +394,31 @@ def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_h
     parts = torch.empty((B * num_heads * splits * (d + 2),), dtype=torch.float32, device=q.device) if splits > 1 else None
     _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
           _opt(parts, "parts"), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], B, num_heads,
-          nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, _stream())
+          nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, int(out_layout), _stream())
 
 
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,
               block_table: torch.Tensor, *, num_heads: int, scale: float, softcap: Optional[float],
-              window: Optional[int], full_precision: bool, kv_layout: int = KV_ROW) -> None:
+              window: Optional[int], full_precision: bool, kv_layout: int = KV_ROW,
+              out_layout: int = LAYOUT_ROW) -> None:
     """Attention of the step's query tokens over the cache; picks the kernel for the step's shape and
     the cache's layout.  `ctx` carries positions, seq_of_token, cu_seqlens, context_lens and the
-    host-side sizes of the step."""
+    host-side sizes of the step.  out_layout FRAG16 is taken by the single-token kernel only."""
     if kv_layout == KV_FRAGMENT:
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
             attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
-                             max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
-        else:
-            attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
-                              num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
-                              max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
+                             max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
+                             out_layout=out_layout)
+            return
+        if out_layout != LAYOUT_ROW:
+            raise HipLibraryError("only the single-token attention kernel writes fragment order")
+        attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
+                          num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
+                          max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
         return
+    if out_layout != LAYOUT_ROW:
+        raise HipLibraryError("only the single-token attention kernel writes fragment order")
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
                       max_position=ctx.max_position, full_precision=full_precision)

@@ -1,4 +1,4 @@
-from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, CacheNeed, KVNeed,
+from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, CacheNeed, FragmentActs, KVNeed,
                    ParamSpec, Part, Precision, Registry, StateNeed)
 from .linear import Linear
 from .stream import ResidualStream

@@ -14,7 +14,7 @@ from typing import Dict, Optional
 import torch
 
 from ..hip import ops
-from .base import MIXERS, CacheNeed, KVNeed, ParamSpec, Part, Precision
+from .base import MIXERS, CacheNeed, FragmentActs, KVNeed, ParamSpec, Part, Precision
 from .linear import Linear
 
 
@@ -71,15 +71,24 @@ class Attention(Part):
     def weight_bytes(self) -> int:
         return self.qkv.nbytes() + self.o.nbytes()
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
-        """x: [T, H] in the activation dtype; returns the branch in float32 ([T, H] or partial sums)."""
+    @property
+    def accepts_fragment_activations(self) -> bool:
+        return self.qkv.accepts_fragment_input
+
+    def forward(self, x, ctx, cache) -> torch.Tensor:
+        """x: [T, H] in the activation dtype (a tensor, or FragmentActs in decode steps); returns the branch
+        in float32 ([T, H] or partial sums)."""
         T = x.shape[0]
         qkv = self.qkv(x, self.precision.act)
         q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
         self.position.rotate_and_store(qkv, q, ctx, cache, num_heads=self.nH, num_kv_heads=self.nKV,
                                        head_dim=self.d, kv_layout=self.kv_layout)
-        out = torch.empty_like(q)
-        ops.attention(q, cache.k, cache.v, out, ctx, cache.block_table, num_heads=self.nH, scale=self.scale,
-                      softcap=self.softcap, window=self.window, full_precision=self.precision.full,
-                      kv_layout=self.kv_layout)
+        # Single tokens on the matrix-core kernel: its output goes to the output projection in fragment order.
+        frag = (getattr(ctx, "fragment_activations", False) and ctx.is_decode and self.kv_layout == ops.KV_FRAGMENT
+                and self.nH // self.nKV <= 16 and self.o.accepts_fragment_input
+                and FragmentActs.possible(self.precision, T, self.q_dim))
+        out = FragmentActs.empty(T, self.q_dim, q.device) if frag else torch.empty_like(q)
+        ops.attention(q, cache.k, cache.v, out.data if frag else out, ctx, cache.block_table, num_heads=self.nH,
+                      scale=self.scale, softcap=self.softcap, window=self.window, full_precision=self.precision.full,
+                      kv_layout=self.kv_layout, out_layout=ops.LAYOUT_FRAG16 if frag else ops.LAYOUT_ROW)
         return self.o(out, torch.float32, allow_partials=True)

@@ -39,6 +39,35 @@ class Precision:
         raise ValueError(f"unknown dtype '{name}': bfloat16 or float32")
 
 
+# --------------------------------------------------------------------------- activations in fragment order
+
+class FragmentActs:
+    """bfloat16 activations [rows, cols] of a decode step (at most 64 rows) stored in the order in which
+    the matrix-core kernels read them ([rows/16][cols/32][64 lanes][8], rows padded to 16): a wave
+    fetches a whole operand with one contiguous read.  Only parts that declare
+    `accepts_fragment_activations` are ever handed one; everything else sees plain tensors."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    @staticmethod
+    def possible(precision: "Precision", rows: int, cols: int) -> bool:
+        return precision.act == torch.bfloat16 and 1 <= rows <= 64 and cols % 32 == 0
+
+    @staticmethod
+    def empty(rows: int, cols: int, device) -> "FragmentActs":
+        padded = -(-rows // 16) * 16
+        return FragmentActs(torch.empty(padded * cols, dtype=torch.bfloat16, device=device), rows, cols)
+
+
 # --------------------------------------------------------------------------- parameters
 
 @dataclass(frozen=True)

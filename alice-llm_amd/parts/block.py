@@ -21,9 +21,13 @@ class SandwichBlock:
         self.norms = norms
 
     def forward(self, stream, ctx, cache) -> None:
-        h = stream.normed(self.norms.get("pre_mixer"))
+        # In decode steps parts that say so take their input in the matrix-core kernels' fragment order.
+        frag = getattr(ctx, "fragment_activations", False)
+        h = stream.normed(self.norms.get("pre_mixer"),
+                          fragments=frag and getattr(self.mixer, "accepts_fragment_activations", False))
         stream.push(self.mixer.forward(h, ctx, cache), self.norms.get("post_mixer"))
-        h = stream.normed(self.norms.get("pre_ff"))
+        h = stream.normed(self.norms.get("pre_ff"),
+                          fragments=frag and getattr(self.feed_forward, "accepts_fragment_activations", False))
         stream.push(self.feed_forward.forward(h, ctx), self.norms.get("post_ff"))
 
 

@@ -71,6 +71,10 @@ class OutputHead(Part):
     def weight_bytes(self) -> int:
         return 0 if self.tied_to else self.proj.nbytes()
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x: [n, dim] normed rows; returns float32 logits [n, V]."""
+    @property
+    def accepts_fragment_activations(self) -> bool:
+        return self.proj.accepts_fragment_input
+
+    def forward(self, x) -> torch.Tensor:
+        """x: [n, dim] normed rows (a tensor or FragmentActs); returns float32 logits [n, V]."""
         return self.proj(x, torch.float32)

@@ -52,6 +52,13 @@ class GatedMLP(Part):
     def weight_bytes(self) -> int:
         return self.gate_up.nbytes() + self.down.nbytes()
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        h = self.gate_up(x, self.precision.act)
+    @property
+    def accepts_fragment_activations(self) -> bool:
+        return self.gate_up.accepts_fragment_input
+
+    def forward(self, x, ctx) -> torch.Tensor:
+        # decode steps: the gated product goes to the down projection in fragment order as well
+        frag = (getattr(ctx, "fragment_activations", False) and self.down.accepts_fragment_input
+                and self.gate_up.can_write_fragments(x.shape[0]))
+        h = self.gate_up(x, self.precision.act, out_fragments=frag)
         return self.down(h, torch.float32, allow_partials=True)

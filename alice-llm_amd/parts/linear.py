@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 from ..hip import ops
-from .base import Precision
+from .base import FragmentActs, Precision
 
 # Whether the bfloat16 path rearranges its weights for the MFMA kernels.  The kernels refuse
 # nothing: shapes they do not cover are padded inside the layout.
@@ -49,17 +49,39 @@ class Linear:
     def nbytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype, *, allow_partials: bool = False,
-                 variant: int = ops.LINEAR_AUTO) -> torch.Tensor:
-        """Returns [M, n], or [S, M, n] float32 partial sums when the kernel prefers to split the
-        inner dimension and the caller can add them up (allow_partials)."""
+    @property
+    def accepts_fragment_input(self) -> bool:
+        """Whether activations in fragment order can be fed in (the MFMA kernels, inner width a multiple of 32)."""
+        return self.layout == ops.LAYOUT_FRAG16 and self.k % 32 == 0
+
+    def can_write_fragments(self, rows: int) -> bool:
+        # the streaming kernel's privilege; very wide outputs go to the tiled kernel from 17 rows on
+        return (self.layout == ops.LAYOUT_FRAG16 and rows <= 64 and self.n % 32 == 0 and not (rows > 16 and self.n >= 65536)
+                and self.epilogue != ops.EPI_SOFTCAP and self.precision.act == torch.bfloat16)
+
+    def __call__(self, x, out_dtype: torch.dtype, *, allow_partials: bool = False,
+                 variant: int = ops.LINEAR_AUTO, out_fragments: bool = False):
+        """x: [M, k] tensor or FragmentActs.  Returns [M, n], or [S, M, n] float32 partial sums when the
+        kernel prefers to split the inner dimension and the caller can add them up (allow_partials), or a
+        FragmentActs when out_fragments is asked for (bfloat16, at most 64 rows)."""
         M = x.shape[0]
+        frag_in = isinstance(x, FragmentActs)
+        if frag_in and not self.accepts_fragment_input:
+            raise ValueError("this projection cannot read activations in fragment order")
         split = 1
         if allow_partials and self.epilogue == ops.EPI_NONE and out_dtype == torch.float32:
             split = ops.linear_split_hint(M, self.n, self.k, self.layout)
-        shape = (split, M, self.n) if split > 1 else (M, self.n)
-        y = torch.empty(shape, dtype=out_dtype, device=x.device)
-        ops.linear(x, self.weight, y, n_out=self.n, k_in=self.k, layout=self.layout,
+        if out_fragments:
+            if not self.can_write_fragments(M) or out_dtype != torch.bfloat16:
+                raise ValueError("this projection cannot write activations in fragment order here")
+            out = FragmentActs.empty(M, self.n, x.device)
+            y = out.data
+        else:
+            shape = (split, M, self.n) if split > 1 else (M, self.n)
+            out = y = torch.empty(shape, dtype=out_dtype, device=x.device)
+        ops.linear(x.data if frag_in else x, self.weight, y, n_out=self.n, k_in=self.k, layout=self.layout,
                    epilogue=self.epilogue, epi_param=self.epi_param, split_k=split, variant=variant,
-                   full_precision=self.precision.full)
-        return y
+                   full_precision=self.precision.full, rows=M,
+                   x_layout=ops.LAYOUT_FRAG16 if frag_in else ops.LAYOUT_ROW,
+                   y_layout=ops.LAYOUT_FRAG16 if out_fragments else ops.LAYOUT_ROW)
+        return out

@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from ..hip import ops
-from .base import Precision
+from .base import FragmentActs, Precision
 
 
 class ResidualStream:
@@ -53,11 +53,25 @@ class ResidualStream:
         self._branch = None
         self._post = None
 
-    def normed(self, norm, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        """Apply the pending add, then return norm(x) in the activation dtype (x itself if norm is None)."""
+    def normed(self, norm, out_dtype: Optional[torch.dtype] = None, fragments: bool = False):
+        """Apply the pending add, then return norm(x) in the activation dtype (x itself if norm is None).
+        fragments: the consumer reads fragment order; given where possible (see FragmentActs), else a tensor."""
         out_dtype = out_dtype or self.precision.act
         T, H = self.x.shape
         pre = norm.fused() if norm is not None and hasattr(norm, "fused") else None
+        if fragments and pre is not None and out_dtype == torch.bfloat16 and FragmentActs.possible(self.precision, T, H):
+            post = self._post
+            pf = post.fused() if post is not None and hasattr(post, "fused") else None
+            if self._branch is not None and not ((post is None or pf is not None) and (pf is None or pf[0].dtype == pre[0].dtype)):
+                self.flush()
+            n, b = self._partials() if self._branch is not None else (1, None)
+            w_post, eps_post, off_post = pf if (pf is not None and b is not None) else (None, 0.0, 0.0)
+            out = FragmentActs.empty(T, H, self.x.device)
+            ops.add_norm(self.x, b, w_post, pre[0], out.data, eps_post=eps_post, eps_pre=pre[1], off_post=off_post,
+                         off_pre=pre[2], n_partials=n, full_precision=self.precision.full, out_layout=ops.LAYOUT_FRAG16)
+            self._branch = None
+            self._post = None
+            return out
         if self._branch is not None and (norm is None or pre is not None):
             post = self._post
             pf = post.fused() if post is not None and hasattr(post, "fused") else None
@@ -78,10 +92,17 @@ class ResidualStream:
             return self.x.to(out_dtype)
         return norm.forward(self.x, out_dtype)
 
-    def rows_normed(self, norm, rows: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def rows_normed(self, norm, rows: torch.Tensor, out_dtype: Optional[torch.dtype] = None, fragments: bool = False):
         """norm(x[rows]) after all pending adds: what the output head reads."""
         self.flush()
         out_dtype = out_dtype or self.precision.act
+        pre = norm.fused() if norm is not None and hasattr(norm, "fused") else None
+        if fragments and pre is not None and out_dtype == torch.bfloat16 and \
+                FragmentActs.possible(self.precision, rows.numel(), self.x.shape[1]):
+            out = FragmentActs.empty(rows.numel(), self.x.shape[1], self.x.device)
+            ops.add_norm(self.x, None, None, pre[0], out.data, eps_pre=pre[1], off_pre=pre[2], rows=rows,
+                         full_precision=self.precision.full, out_layout=ops.LAYOUT_FRAG16)
+            return out
         if norm is None:
             return self.x.index_select(0, rows.long()).to(out_dtype)
         return norm.forward(self.x, out_dtype, rows=rows)

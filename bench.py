@@ -116,7 +116,7 @@ def main() -> int:
         eng = model.engine(max_tokens=args.context, max_seqs=1)
         p = prompts(1)
         times = []
-        for it in range(3):
+        for it in range(6):
             s = eng.open(1)
             sync()
             t = time.perf_counter()

@@ -381,6 +381,102 @@ def test_linear_mfma_rows_do_not_depend_on_the_batch():
         assert torch.equal(run(x[:33].contiguous(), variant), full[:33])
 
 
+def acts_to_fragments(x):
+    """Activations [M, K] (K a multiple of 32) in fragment order, written out in plain indexing:
+    [M/16][K/32][lane = g*16 + r][8] holds x[16 mt + r][32 kt + 8 g + e]; rows padded with NaN so that a
+    kernel that lets a padded row into a real one shows."""
+    M, K = x.shape
+    Mp = -(-M // 16) * 16
+    xp = torch.full((Mp, K), float("nan"), dtype=x.dtype)
+    xp[:M] = x.cpu()
+    return xp.view(Mp // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1).to(DEV)
+
+
+def acts_from_fragments(flat, M, K):
+    Mp = -(-M // 16) * 16
+    return flat.cpu().view(Mp // 16, K // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(Mp, K)[:M]
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 224, 160), (16, 4096, 256), (17, 160, 320), (33, 64, 96), (64, 2304, 1024),
+                                   (40, 65536 + 32, 64)])
+def test_linear_mfma_activations_in_fragment_order(M, N, K):
+    x, w = rnd(M, K, seed=16, dtype=torch.bfloat16), rnd(N, K, seed=17, scale=0.1, dtype=torch.bfloat16)
+    wf, xf = ops.to_frag16(w), acts_to_fragments(x)
+    assert torch.equal(acts_from_fragments(xf, M, K), x.cpu())
+    row = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, wf, row, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False)
+    close(row, x.double() @ w.double().T, 1e-2 * math.sqrt(K / 64), 2 ** -8)
+    # reading fragments, writing rows: the same bits as from rows (float32 partial sums too)
+    y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(xf, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16)
+    assert torch.equal(y, row)
+    if N < 65536:
+        for split in (1, 2):
+            shape = (split, M, N) if split > 1 else (M, N)
+            a, b = torch.empty(shape, device=DEV), torch.empty(shape, device=DEV)
+            ops.linear(x, wf, a, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False)
+            ops.linear(xf, wf, b, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False, rows=M,
+                       x_layout=ops.LAYOUT_FRAG16)
+            assert torch.equal(a, b)
+        # writing fragments (the streaming kernel only)
+        for src, lay in ((x, ops.LAYOUT_ROW), (xf, ops.LAYOUT_FRAG16)):
+            yf = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ops.linear(src, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, x_layout=lay,
+                       y_layout=ops.LAYOUT_FRAG16)
+            assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
+    else:
+        yf = torch.empty((-(-M // 16) * 16) * N, dtype=torch.bfloat16, device=DEV)
+        with pytest.raises(ops.HipLibraryError, match="fragment order"):
+            ops.linear(x, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, y_layout=ops.LAYOUT_FRAG16)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 96, 96)])
+def test_linear_mfma_geglu_in_fragment_order(M, N, K):
+    x, w = rnd(M, K, seed=18, dtype=torch.bfloat16), rnd(2 * N, K, seed=19, scale=0.3, dtype=torch.bfloat16)
+    wf, xf = ops.to_frag16(w), acts_to_fragments(x)
+    row = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, wf, row, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, full_precision=False)
+    yf = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(xf, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, full_precision=False, rows=M,
+               x_layout=ops.LAYOUT_FRAG16, y_layout=ops.LAYOUT_FRAG16)
+    assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
+
+
+def test_linear_refuses_fragment_order_it_cannot_take():
+    x, w = rnd(8, 40, seed=1, dtype=torch.bfloat16), rnd(48, 40, seed=2, dtype=torch.bfloat16)
+    y = torch.empty(8, 48, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.HipLibraryError, match="K % 32"):      # inner width no multiple of 32
+        ops.linear(torch.empty(16 * 40, dtype=torch.bfloat16, device=DEV), ops.to_frag16(w), y, n_out=48, k_in=40,
+                   layout=ops.LAYOUT_FRAG16, full_precision=False, rows=8, x_layout=ops.LAYOUT_FRAG16)
+    w2 = rnd(48, 64, seed=2, dtype=torch.bfloat16)
+    with pytest.raises(ops.HipLibraryError, match="fragment order"):    # output width no multiple of 32
+        ops.linear(rnd(8, 64, dtype=torch.bfloat16), ops.to_frag16(w2), torch.empty(16 * 48, dtype=torch.bfloat16, device=DEV),
+                   n_out=48, k_in=64, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=8, y_layout=ops.LAYOUT_FRAG16)
+    with pytest.raises(ops.HipLibraryError, match="generic kernel"):   # the 32-bit path has rows only
+        ops.linear(torch.empty(16 * 64, dtype=torch.bfloat16, device=DEV), w2, y, n_out=48, k_in=64, full_precision=True, rows=8,
+                   x_layout=ops.LAYOUT_FRAG16)
+
+
+@pytest.mark.parametrize("T,H", [(1, 64), (8, 2304), (37, 96), (64, 4608), (20, 10016)])
+def test_add_norm_writes_fragment_order(T, H):
+    x0, br = rnd(T, H, seed=2, scale=3.0), rnd(2, T, H, seed=3, scale=0.5)
+    wp, wq = rnd(H, seed=4, scale=0.1, dtype=torch.bfloat16), rnd(H, seed=5, scale=0.1, dtype=torch.bfloat16)
+    xa, xb = x0.clone(), x0.clone()
+    row = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    ops.add_norm(xa, br, wp, wq, row, eps_post=1e-6, eps_pre=1e-5, off_post=1.0, off_pre=1.0, n_partials=2, full_precision=False)
+    flat = torch.full(((-(-T // 16) * 16) * H,), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.add_norm(xb, br, wp, wq, flat, eps_post=1e-6, eps_pre=1e-5, off_post=1.0, off_pre=1.0, n_partials=2, full_precision=False,
+                 out_layout=ops.LAYOUT_FRAG16)
+    assert torch.equal(xa, xb) and torch.equal(acts_from_fragments(flat, T, H), row.cpu())
+    # gathered rows (what the output head reads)
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32, device=DEV)
+    row = torch.empty(3, H, dtype=torch.bfloat16, device=DEV)
+    ops.add_norm(xa, None, None, wq, row, eps_pre=1e-5, off_pre=1.0, rows=rows, full_precision=False)
+    flat = torch.empty(16 * H, dtype=torch.bfloat16, device=DEV)
+    ops.add_norm(xa, None, None, wq, flat, eps_pre=1e-5, off_pre=1.0, rows=rows, full_precision=False, out_layout=ops.LAYOUT_FRAG16)
+    assert torch.equal(acts_from_fragments(flat, 3, H), row.cpu())
+
+
 def test_embed_from_fragment_layout():
     V, H = 301, 72
     table = rnd(V, H, seed=1, dtype=torch.bfloat16)
@@ -463,6 +559,13 @@ def test_attention_mfma_single_tokens(nH, nKV, d, cap, window):
         ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=cap,
                              window=window, splits=splits)
         close(out, ref, 2e-2)
+    # output in fragment order for the projection that follows: the same bits, elsewhere
+    if (nH * d) % 32 == 0:
+        ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=cap, window=window)
+        flat = torch.full((16 * nH * d,), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_decode(q, kp, vp, flat, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=cap,
+                             window=window, out_layout=ops.LAYOUT_FRAG16)
+        assert torch.equal(acts_from_fragments(flat, len(lens), nH * d), out.cpu())
     # the prompt kernels on single tokens give the same
     for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT):
         out = torch.full_like(q, float("nan"))
