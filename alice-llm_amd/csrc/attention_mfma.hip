@@ -452,21 +452,36 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// Combines the splits of one (sequence, head) in the order 0, 1, ...: grid (sequences * heads), D threads.
+// Combines the splits of one (sequence, head): grid (sequences * heads).  The first wave fetches every
+// split's maximum and sum at once and leaves the weights in LDS; then each thread sums its elements over the
+// splits in the order 0, 1, ..., eight loads in flight at a time (a loop of dependent round trips to memory
+// would cost more than the arithmetic).
 __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits,
                                           int nH, int out_layout) {
+  __shared__ float fs[65];
   const float* pr = parts + (size_t)blockIdx.x * splits * (D + 2);
-  float mm = -INFINITY;
-  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, pr[(size_t)s * (D + 2)]);
-  for (int e = threadIdx.x; e < D; e += blockDim.x) {
-    float acc = 0.f, ll = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float* ps = pr + (size_t)s * (D + 2);
-      const float f = (ps[0] == -INFINITY) ? 0.f : exp2_fast(ps[0] - mm);
-      acc += ps[2 + e] * f;
-      ll += ps[1] * f;
+  const int t = threadIdx.x;
+  if (t < 64) {
+    const float m = t < splits ? pr[(size_t)t * (D + 2)] : -INFINITY;
+    const float l = t < splits ? pr[(size_t)t * (D + 2) + 1] : 0.f;
+    const float mm = wave_max(m);
+    const float f = (m == -INFINITY) ? 0.f : exp2_fast(m - mm);
+    const float ll = wave_sum(l * f);
+    fs[t] = f;
+    if (t == 0) fs[64] = ll;
+  }
+  __syncthreads();
+  const float inv = 1.f / fs[64];
+  for (int e = t; e < D; e += blockDim.x) {
+    float acc = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int p = 0; p < 8; ++p) v[p] = (s0 + p < splits) ? pr[(size_t)(s0 + p) * (D + 2) + 2 + e] : 0.f;
+#pragma unroll
+      for (int p = 0; p < 8; ++p) acc += v[p] * fs[min(s0 + p, 63)];
     }
-    out[decode_out_index(out_layout, blockIdx.x / nH, (blockIdx.x % nH) * D + e, nH * D)] = f32_to_bf16(acc / ll);
+    out[decode_out_index(out_layout, blockIdx.x / nH, (blockIdx.x % nH) * D + e, nH * D)] = f32_to_bf16(acc * inv);
   }
 }
 

@@ -209,6 +209,8 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
   if (H <= 1024) { threads = 256; ept = H <= 256 ? 1 : (H <= 512 ? 2 : 4); }
   else if (H <= 4096) { threads = 1024; ept = 4; }
   else if (H <= 8192) { threads = 1024; ept = 8; }
+  // Many rows: smaller blocks with more elements a thread keep more rows and more loads in flight on a CU.
+  if (T >= 256 && H > 1024 && H <= 4096) { threads = H <= 2048 ? 256 : 512; ept = 8; }
 #define ARGS resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, \
              eps_post, eps_pre, off_post, off_pre, out_layout
 #define LAUNCH(TW, TO, FULL)                                                                         \

@@ -454,11 +454,22 @@ extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStre
 
 int alice_linear_split_hint_frag(int M, int N, int K) {
   if (M > 64) {
-    // Tiled kernel: 128 tokens x 256 features a block.  Narrow outputs leave most of the chip idle: halve
-    // or quarter the inner dimension instead of the tile.
+    // Tiled kernel: 128 tokens x 256 features a block, two blocks a CU.  Narrow outputs leave most of the
+    // chip idle; slices of the inner dimension fill it.  Cost of s slices, relative to one block a CU
+    // running the whole inner dimension: the busiest CU runs n = ceil(blocks s / 256) blocks of 1/s the
+    // length, two at a time at 1.7 times the time of one; every extra slice writes and reads another
+    // [M, N] float32 partial result (both constants fitted to measurements at N = 2304, K = 2048 and 9216).
     const int blocks = ceil_div(N, 256) * ceil_div(M, 128), KT = (K + 31) / 32;
-    if (blocks >= 200 || KT < 32) return 1;
-    return 2;
+    if (blocks >= 384) return 1;
+    int best = 1;
+    float best_cost = 1e30f;
+    for (int s = 1; s <= 6; ++s) {
+      if (s > 1 && KT / s < 16) break;
+      const int n = ceil_div(blocks * s, 256);
+      const float cost = (1.7f * (n / 2) + (n % 2)) / s + 3.6f * blocks / K * (s - 1);
+      if (cost < best_cost * 0.97f) { best_cost = cost; best = s; }
+    }
+    return best;
   }
   const int KT = (K + 31) / 32;
   if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);

@@ -138,16 +138,17 @@ def fill_pools(kp, vp, bt, k, v, seq, start=0):
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nH,nKV,d,R", [(4, 1, 16, 16), (6, 3, 24, 24), (2, 2, 40, 16), (3, 1, 256, 256)])
-def test_rope_cache_write(dt, nH, nKV, d, R):
-    lens, starts = [5, 70, 1], [0, 60, 130]
+@pytest.mark.parametrize("many", [False, True])      # few tokens and many take different kernels
+def test_rope_cache_write(dt, nH, nKV, d, R, many):
+    lens, starts = ([5, 270, 1], [0, 60, 130]) if many else ([5, 70, 1], [0, 60, 130])
     T = sum(lens)
     qkv = rnd(T, (nH + 2 * nKV) * d + 8, seed=10, dtype=DT[dt])[:, :].contiguous()       # rows longer than the heads
     pos = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32, device=DEV)
     seq = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
-    kp, vp, bt = paged(192, nKV, d, DT[dt], 3, seed=11)
+    kp, vp, bt = paged(384, nKV, d, DT[dt], 3, seed=11)
     theta = 5e5
     j = torch.arange(R // 2, dtype=D)
-    ang = torch.arange(200, dtype=D)[:, None] * theta ** (-2.0 * j / R)
+    ang = torch.arange(400, dtype=D)[:, None] * theta ** (-2.0 * j / R)
     cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
     q_out = torch.empty(T, nH * d, dtype=DT[dt], device=DEV)
     ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
@@ -535,6 +536,41 @@ def test_fragment_cache_layout_is_what_the_comment_says():
         w = tp % 16
         voff = (((tp // 32) * (d // 16) + e // 16) * 64 + (w // 4) * 16 + e % 16) * 8 + (((tp % 32) // 16) * 4 + w % 4)
         assert kflat[koff] == k[t, h, e] and vflat[voff] == v[t, h, e]
+
+
+@pytest.mark.parametrize("nH,nKV,d", [(3, 2, 64), (8, 4, 256), (2, 1, 128), (1, 1, 32)])
+def test_rope_into_the_fragment_cache_layout(nH, nKV, d):
+    # rotation and the fragment layout together, every element checked through the layout's formula
+    _rope_fragment_case(nH, nKV, d, [70, 3], [0, 62])
+    _rope_fragment_case(nH, nKV, d, [290, 3], [0, 62])       # many tokens: the vector kernel
+
+
+def _rope_fragment_case(nH, nKV, d, lens, starts):
+    T = sum(lens)
+    qkv = rnd(T, (nH + 2 * nKV) * d, seed=40, dtype=torch.bfloat16)
+    pos = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    kp, vp, bt = paged(320, nKV, d, torch.bfloat16, 2, seed=41)
+    theta = 1e4
+    ang = torch.arange(300, dtype=D)[:, None] * theta ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    q_out = torch.empty(T, nH * d, dtype=torch.bfloat16, device=DEV)
+    ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                         rotary_dim=d, max_position=int(pos.max()), kv_layout=ops.KV_FRAGMENT)
+    x = qkv.double().cpu()
+    q = P.rope_half_split(x[:, :nH * d].view(T, nH, d), pos.cpu(), theta)
+    k = P.rope_half_split(x[:, nH * d:(nH + nKV) * d].view(T, nKV, d), pos.cpu(), theta)
+    v = x[:, (nH + nKV) * d:].view(T, nKV, d)
+    close(q_out.view(T, nH, d), q, 2 ** -5, 2 ** -7)
+    e = torch.arange(d)
+    for t in range(T):
+        page, tp = int(bt[int(seq[t]), int(pos[t]) // 64]), int(pos[t]) % 64
+        koff = (((tp // 16) * (d // 32) + e // 32) * 64 + ((e % 32) // 8) * 16 + tp % 16) * 8 + e % 8
+        w = tp % 16
+        voff = (((tp // 32) * (d // 16) + e // 16) * 64 + (w // 4) * 16 + e % 16) * 8 + (((tp % 32) // 16) * 4 + w % 4)
+        for h in range(nKV):
+            close(kp[page, h].reshape(-1).cpu()[koff], k[t, h], 2 ** -5, 2 ** -7)
+            assert torch.equal(vp[page, h].reshape(-1).cpu()[voff].double(), v[t, h])
 
 
 @pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
