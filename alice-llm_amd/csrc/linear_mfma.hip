@@ -362,7 +362,7 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   dim3 grid(groups, split);
   // Eight waves a block when the slice is long enough to give each of them work and the block count is
   // too low to fill the chip with four.
-  const bool eight = (RT * MT <= 8) && per >= 32 && groups * split < 2048;
+  const bool eight = (RT * MT <= 4) && per >= 32 && groups * split < 2048;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
     linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, x_frag, y_frag);
@@ -375,21 +375,21 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
 }
 
 // Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
-// on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)
-int skinny_row_tiles(int M, int N, int epi, int split) {
+// on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)  Measured on the 2B
+// shapes with the activations in fragment order.
+int skinny_row_tiles(int M, int N, int epi, int split, int K) {
   const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   if (tiles >= 4096) return 4;
-  // Many tokens: more rows per block per read of the activations, wherever the inner dimension can be
-  // split over blocks to keep the chip busy (measured on the 2B shapes).
-  if (M > 32 && (tiles >= 1024 || (split > 1 && tiles >= 64))) return 4;
-  if (tiles >= 1024 || epi == ALICE_EPI_GEGLU) return 2;
-  return 1;
+  if (epi == ALICE_EPI_GEGLU) return 2;
+  // Many tokens and slices of the inner dimension: more rows per block per read of the activations.
+  if (M > 32 && split > 1 && tiles >= 64) return K >= 8192 ? 4 : 2;
+  return tiles >= 1024 ? 2 : 1;
 }
 
 template <int EPI, typename TO>
 int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
                     hipStream_t s) {
-  const int rt = skinny_row_tiles(M, N, EPI, split);
+  const int rt = skinny_row_tiles(M, N, EPI, split, K);
 #define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, x_frag, y_frag, s)
 #define BY_RT(MT)                                                   \
   do {                                                              \
@@ -473,7 +473,7 @@ int alice_linear_split_hint_frag(int M, int N, int K) {
   }
   const int KT = (K + 31) / 32;
   if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);
-  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE, 1));
+  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE, 1, K));
   int split = 1;
   // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
   while (groups * split < 1024 && KT / (split * 2) >= 16 && split < 16) split *= 2;
