@@ -26,6 +26,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
+// A weight fragment of zeros: k-tiles beyond a slice read it instead of the matrix, so that every load of
+// the main loops is unconditional and nothing has to be patched after a load.
+// (Not declared const: that would put it into the constant address space, and a pointer that may point
+// into either space is dereferenced with the slower flat loads.)
+__device__ __align__(16) uint32_t g_zero_tile[256];
+
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
 }
@@ -84,10 +90,15 @@ __device__ __forceinline__ void store4_frag(bf16_t* __restrict__ y, int m, int n
 // waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
 // tiles (for GeGLU: RT/2 gate tiles and the RT/2 up tiles that belong to them); grid.y: slices of the
 // inner dimension, each writing its own partial sum y[slice][M][N] (slices > 1 only without epilogue).
-template <int RT, int MT, int NW, int EPI, typename TO, bool FULL>
+//
+// Every load of the main loop is unconditional: addresses beyond the matrix or the slice are clamped to
+// valid ones and what they bring is replaced by zeros (weights) or lands in output columns that are never
+// stored (tokens beyond M).  Only then does the compiler know how many loads are in flight and wait for the
+// oldest alone (s_waitcnt vmcnt(n)); a load under a branch makes it wait for all of them.
+template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                            int kt_per_slice, float epi, int x_frag, int y_frag) {
+                                                            int kt_per_slice, float epi, int y_frag) {
   extern __shared__ __align__(16) float red[];            // [NW - 1][RT*MT][64][4]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -99,7 +110,10 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
     if (EPI == ALICE_EPI_GEGLU) tile[i] = (i & 1) ? (N / 16 + blockIdx.x * (RT / 2) + (i >> 1)) : (blockIdx.x * (RT / 2) + (i >> 1));
     else tile[i] = blockIdx.x * RT + i;
   }
-  const int tile_limit = NT;
+  // where this lane reads its weight fragments (rows beyond the matrix: the last tile's, results unused)
+  const bf16_t* wrow[RT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i) wrow[i] = wf + (size_t)min(tile[i], NT - 1) * KT * 512 + lane * 8;
   f32x4 acc[RT][MT];
 #pragma unroll
   for (int i = 0; i < RT; ++i)
@@ -108,25 +122,35 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
 
   bool row_ok[MT];
   int row[MT];
+  const bf16_t* xrow[MT];        // this lane's place in the activations at k-tile 0
 #pragma unroll
-  for (int j = 0; j < MT; ++j) { row[j] = j * 16 + r; row_ok[j] = row[j] < M; }
+  for (int j = 0; j < MT; ++j) {
+    row[j] = j * 16 + r;
+    row_ok[j] = row[j] < M;
+    if constexpr (XF) xrow[j] = x + ((size_t)min(j, (M - 1) >> 4) * KT * 64 + lane) * 8;
+    else xrow[j] = x + (size_t)min(row[j], M - 1) * K;
+  }
 
   // A rolling window of U k-tiles per wave: wave w takes k-tiles kb + w, kb + w + NW, ...; as soon as a
   // tile's fragments have gone into the MFMAs their registers are refilled with the tile U steps ahead,
   // so U loads per operand stay in flight all the time.
   constexpr int U = (RT * MT >= 8) ? 3 : 4;
   u32x4 a[U][RT], b[U][MT];
+  const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
   auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
     const bool kok = kt < ke;
+    const int ktc = kok ? kt : 0;                           // past the slice: zero weights, any activations
 #pragma unroll
-    for (int i = 0; i < RT; ++i) {
-      aa[i] = u32x4{0u, 0u, 0u, 0u};
-      if (kok && tile[i] < tile_limit)
-        aa[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
+    for (int i = 0; i < RT; ++i) aa[i] = *reinterpret_cast<const u32x4*>(kok ? wrow[i] + (size_t)ktc * 512 : zero);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      if constexpr (XF) {
+        bb[j] = *reinterpret_cast<const u32x4*>(xrow[j] + (size_t)ktc * 512);
+      } else {
+        // a row's last, partial k-tile: the weights are zero there, so any finite values do
+        bb[j] = *reinterpret_cast<const u32x4*>(xrow[j] + min(ktc * 32 + g * 8, K - 8));
+      }
     }
-#pragma unroll
-    for (int j = 0; j < MT; ++j)
-      bb[j] = x_frag ? load_x_frag_f(x, j, kok, KT, kt, lane) : load_x_frag(x, row[j], row_ok[j] && kok, K, kt, g);
   };
   // Blocks start at different places of their k range and wrap around: all blocks read the same
   // activations, and in lockstep they would all ask the same L2 channel for the same line at once.
@@ -138,16 +162,31 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
     return t < J ? kb + wave + j * NW : ke;                 // past the sequence: nothing to load
   };
 #pragma unroll
-  for (int u = 0; u < U; ++u) fetch(tile_at(u), a[u], b[u]);
-  for (int t0 = 0; t0 < J; t0 += U) {
+  for (int u = 0; u < U; ++u) {
+    fetch(tile_at(u), a[u], b[u]);
+    __builtin_amdgcn_sched_barrier(0);       // slot by slot, oldest first: the loop waits for the oldest only
+  }
+  for (int t0 = 0; t0 + U < J; t0 += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < MT; ++j) acc[i][j] = mfma16(a[u][i], b[u][j], acc[i][j]);
-      fetch(tile_at(t0 + U + u), a[u], b[u]);      // tiles past the end come back as zeros
+      // The refill is issued here, U - 1 steps ahead of its use: the scheduler must not move it down to
+      // the use (it would, to save registers).
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(tile_at(t0 + U + u), a[u], b[u]);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  }
+  // the last window: nothing is left to fetch (slots past the end hold zero weights)
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) acc[i][j] = mfma16(a[u][i], b[u][j], acc[i][j]);
   }
 
   if (wave > 0) {
@@ -244,9 +283,17 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
       tile[i] = (bx * 4 + wave) * WN + i;
     }
   }
-  int xrow[XJ];
+  // Loads are unconditional (see the streaming kernel): rows and tiles beyond the matrix are clamped, and
+  // k-tiles beyond the slice bring zero weights.
+  const bf16_t* xsrc[XJ];        // this lane's place in the activations at k-tile 0, for the token tiles it stages
 #pragma unroll
-  for (int j = 0; j < XJ; ++j) xrow[j] = min(m0 + (XJ * wave + j) * 16 + r, M - 1);
+  for (int j = 0; j < XJ; ++j) {
+    if constexpr (XF) xsrc[j] = x + ((size_t)min((m0 >> 4) + XJ * wave + j, (M - 1) >> 4) * KT * 64 + lane) * 8;
+    else xsrc[j] = x + (size_t)min(m0 + (XJ * wave + j) * 16 + r, M - 1) * K;
+  }
+  const bf16_t* wsrc[WN];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) wsrc[i] = wf + (size_t)min(tile[i], NT - 1) * KT * 512 + lane * 8;
 
   f32x4 acc[WN][TM];
 #pragma unroll
@@ -261,9 +308,9 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
     for (int kc = 0; kc < KC; ++kc)
 #pragma unroll
       for (int j = 0; j < XJ; ++j) {
-        const int kt = kt_base + s * KC + kc;
-        if constexpr (XF) xr[kc][j] = load_x_frag_f(x, min((m0 >> 4) + XJ * wave + j, (M - 1) >> 4), kt < kt_end, KT, kt, lane);
-        else xr[kc][j] = load_x_frag(x, xrow[j], kt < kt_end, K, kt, g);
+        const int kt = max(0, min(kt_base + s * KC + kc, kt_end - 1));      // past the slice: the weights are zeros
+        if constexpr (XF) xr[kc][j] = *reinterpret_cast<const u32x4*>(xsrc[j] + (size_t)kt * 512);
+        else xr[kc][j] = *reinterpret_cast<const u32x4*>(xsrc[j] + min(kt * 32 + g * 8, K - 8));
       }
   };
   auto stage_store = [&](int buf) {
@@ -272,13 +319,12 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
 #pragma unroll
       for (int j = 0; j < XJ; ++j) xs[((buf * KC + kc) * TM + XJ * wave + j) * 64 + lane] = xr[kc][j];
   };
+  const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
   auto w_load = [&](int rel, u32x4 (&w)[WN]) {                // rel: k-tile relative to the slice
     const int kt = kt_base + rel;
+    const bool kok = kt < kt_end;
 #pragma unroll
-    for (int i = 0; i < WN; ++i) {
-      w[i] = u32x4{0u, 0u, 0u, 0u};
-      if (tile[i] < NT && kt < kt_end) w[i] = *reinterpret_cast<const u32x4*>(wf + ((size_t)tile[i] * KT + kt) * 512 + lane * 8);
-    }
+    for (int i = 0; i < WN; ++i) w[i] = *reinterpret_cast<const u32x4*>(kok ? wsrc[i] + (size_t)kt * 512 : zero);
   };
   // blockIdx.y: the slice of the inner dimension this block sums (its own partial result y[slice][M][N])
   const int kt_lo = blockIdx.y * kt_per_slice, kt_hi = min(KT, kt_lo + kt_per_slice);
@@ -287,10 +333,14 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
   stage_load(0);
   stage_store(0);
 #pragma unroll
-  for (int kc = 0; kc < KC; ++kc) w_load(kc, wk[kc]);
-  for (int s = 0; s < S; ++s) {
-    if (s + 1 < S) stage_load(s + 1);
-    __syncthreads();
+  for (int kc = 0; kc < KC; ++kc) {
+    w_load(kc, wk[kc]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // Loads run one stage ahead and are unconditional (a k-tile beyond the slice in the last, partial stage
+  // reads the zero tile); the scheduling barriers keep them where they are issued, so that each wait is for
+  // the oldest loads only.
+  auto stage_mfma = [&](int s, bool more) {
     u32x4 xf[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC) * TM + j) * 64 + lane];
@@ -303,10 +353,24 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
         // this token tile's fragment has had its last use: read the next k-tile's into the same registers
         if (kc + 1 < KC) xf[j] = xs[(((s & 1) * KC + kc + 1) * TM + j) * 64 + lane];
       }
-      // this k-tile's weight registers are free again: fetch the same slot of the next stage
-      if (s + 1 < S) w_load((s + 1) * KC + kc, wk[kc]);
+      if (more) {
+        // this k-tile's weight registers are free again: fetch the same slot of the next stage
+        __builtin_amdgcn_sched_barrier(0);
+        w_load((s + 1) * KC + kc, wk[kc]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    if (s + 1 < S) stage_store((s + 1) & 1);
+  };
+  for (int s = 0; s + 1 < S; ++s) {
+    stage_load(s + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    stage_mfma(s, true);
+    stage_store((s + 1) & 1);
+  }
+  if (S > 0) {                   // the last stage has nothing to fetch
+    __syncthreads();
+    stage_mfma(S - 1, false);
   }
 
 #pragma unroll
@@ -365,10 +429,12 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   const bool eight = (RT * MT <= 4) && per >= 32 && groups * split < 2048;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
-    linear_skinny_kernel<RT, MT, 8, EPI, TO, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, x_frag, y_frag);
+    if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
+    else linear_skinny_kernel<RT, MT, 8, EPI, TO, false, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
   } else {
     const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-    linear_skinny_kernel<RT, MT, 4, EPI, TO, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, x_frag, y_frag);
+    if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
+    else linear_skinny_kernel<RT, MT, 4, EPI, TO, false, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
   }
   ALICE_LAUNCH_CHECK();
   return 0;
