@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
     const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
   constexpr int D = DT * 32;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
   const int group = nH / nKV, passes = (group + GH - 1) / GH;
   const int b = blockIdx.y, kvh = blockIdx.z / passes, h0 = (blockIdx.z % passes) * GH;
@@ -230,8 +230,10 @@ __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
   if constexpr (GH == 1) {
     // Two waves per SIMD (256 registers each) hide each other's waits.  Keys and the first half of the values
     // are fetched together; the second half of the values goes into the registers that the keys leave.
+    int page_next = kb_begin <= kb_end ? bt[kb_begin >> 1] : 0;     // one block ahead, through the scalar cache
     for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
-      const int page = bt[kb32 >> 1];
+      const int page = page_next;
+      page_next = bt[min(kb32 + 1, kb_end) >> 1];
       const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems + ((size_t)(kb32 & 1) * 2 * DT * 64 + lane) * 8;
       u32x4 kf[2][DT], va[DT], vb[DT], p[1];
       Core<DT, GH>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
   constexpr int D = DT * 32;
   __shared__ float sm[4][16], sl[4][16];
   extern __shared__ __align__(16) float so[];                // [3 waves][16 columns][D + 4]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
   const int group = nH / nKV;
   const int b = blockIdx.y, head = blockIdx.z, kvh = head / group;
@@ -309,8 +311,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
       if (tok_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
     }
   }
+  // The page number of the next block of keys is read (through the scalar cache: the whole wave asks for the
+  // same one) while this block is computed.
+  int page_next = my_first <= my_last ? bt[my_first >> 1] : 0;
   for (int kb32 = my_first; kb32 <= my_last; ++kb32) {
-    const int page = bt[kb32 >> 1];
+    const int page = page_next;
+    page_next = bt[min(kb32 + 1, my_last) >> 1];
     const bf16_t* vp = v_pool + ((size_t)page * nKV + kvh) * page_elems + ((size_t)(kb32 & 1) * 2 * DT * 64 + lane) * 8;
     u32x4 kf[2][DT], va[DT], vb[DT], p[1];
     Core<DT, 1>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
@@ -375,7 +381,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   constexpr int D = DT * 32;
   __shared__ float sm[4][16], sl[4][16];
   extern __shared__ __align__(16) float so[];            // [4 waves][group][D + 4]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
   const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int group = nH / nKV;
@@ -403,19 +409,28 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
   }
   // Two sets of fragment registers: while one block of keys is computed, the next one's loads are in flight.
+  // The page numbers are read one step before the tiles they name, through the scalar cache (the indices are
+  // the same for the whole wave): a wait for them is no wait for the tiles in flight.
   {
     u32x4 kf0[2][DT], vf0[2 * DT], kf1[2][DT], vf1[2 * DT];
-    auto fetch = [&](int kb32, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
-      const int page = bt[kb32 >> 1];
+    auto page_of = [&](int kb32) { return bt[min(kb32, my_last) >> 1]; };
+    auto fetch = [&](int kb32, int page, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
       Core<DT, 1>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
       Core<DT, 1>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
     };
-    if (my_first <= my_last) fetch(my_first, kf0, vf0);
+    int page_a = 0, page_b = 0;
+    if (my_first <= my_last) {
+      page_a = page_of(my_first);
+      page_b = page_of(my_first + 1);
+      fetch(my_first, page_a, kf0, vf0);
+    }
     for (int kb32 = my_first; kb32 <= my_last; kb32 += 2) {
-      if (kb32 + 1 <= my_last) fetch(kb32 + 1, kf1, vf1);
+      if (kb32 + 1 <= my_last) fetch(kb32 + 1, page_b, kf1, vf1);
+      page_a = page_of(kb32 + 2);
+      page_b = page_of(kb32 + 3);
       c.template compute<SOFTCAP>(kf0, vf0, kb32 << 5, cpos, window, sc, lane);
       if (kb32 + 1 <= my_last) {
-        if (kb32 + 2 <= my_last) fetch(kb32 + 2, kf0, vf0);
+        if (kb32 + 2 <= my_last) fetch(kb32 + 2, page_a, kf0, vf0);
         c.template compute<SOFTCAP>(kf1, vf1, (kb32 + 1) << 5, cpos, window, sc, lane);
       }
     }
