@@ -119,43 +119,84 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const float* __restri
     store_f32(o, out_index(out_layout, r, i, H), x[i] * inv * (off_pre + load_f32(w_pre, i)));
 }
 
-// The same operation with a row held in registers (EPT elements per thread): every operand is read
-// once and the three phases need no second trip through memory.  Used when the row fits.
+// The same operation with a row held in registers (EPT elements per thread): every operand is read once
+// and the three phases need no second trip through memory.  Used when the row fits.
+//
+// All loads come first, unconditionally (indices beyond the row are clamped to its last element and the
+// values replaced by zeros afterwards; the launch leaves few such threads), and nothing is converted or
+// used before the last one is issued: the operands are a few hundred KB that other kernels have just
+// written, they come from memory, and every load that waits for an earlier one costs a round trip.
+template <typename T> struct raw_of;
+template <> struct raw_of<float> { typedef float type; };
+template <> struct raw_of<bf16_t> { typedef uint16_t type; };
+__device__ __forceinline__ float raw_to_f32(float v) { return v; }
+__device__ __forceinline__ float raw_to_f32(uint16_t v) { return bf16_bits_to_f32(v); }
+
+template <int EPT, int C, int CMAX>
+__device__ __forceinline__ void load_partials(float (&t)[EPT][CMAX], const float* __restrict__ row, const int (&idx)[EPT],
+                                              int p0, int n_partials, size_t partial_stride) {
+#pragma unroll
+  for (int j = 0; j < EPT; ++j)
+#pragma unroll
+    for (int p = 0; p < C; ++p) t[j][p] = row[idx[j] + (size_t)min(p0 + p, n_partials - 1) * partial_stride];
+}
+
 template <typename TW, typename TO, bool FULL, int EPT>
 __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __restrict__ branch,
                                      int n_partials, size_t partial_stride,
                                      const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
                                      TO* __restrict__ out, const int* __restrict__ rows, int H,
                                      float eps_post, float eps_pre, float off_post, float off_pre, int out_layout) {
+  typedef typename raw_of<TW>::type RW;
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t src = (size_t)(rows ? rows[r] : r) * H;
-  float xv[EPT], bv[EPT], wq[EPT];
+  int idx[EPT];
+  bool in_row[EPT];
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int i = threadIdx.x + j * blockDim.x;
-    xv[j] = i < H ? resid[src + i] : 0.f;
-    wq[j] = (w_pre && i < H) ? load_f32(w_pre, i) : 0.f;
+    in_row[j] = i < H;
+    idx[j] = min(i, H - 1);
+  }
+  // ---- loads
+  constexpr int CMAX = EPT >= 8 ? 4 : 8;        // partial sums in flight per element (registers)
+  float xv[EPT], bv[EPT], t[EPT][CMAX];
+  RW wq_raw[EPT], wp_raw[EPT];
+  const int chunk = n_partials <= 1 ? 1 : (n_partials <= 2 ? 2 : (n_partials <= 4 ? 4 : CMAX));
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) xv[j] = resid[src + idx[j]];
+  if (w_pre) {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) wq_raw[j] = reinterpret_cast<const RW*>(w_pre)[idx[j]];
+  }
+  if (branch) {
+    if (w_post) {
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) wp_raw[j] = reinterpret_cast<const RW*>(w_post)[idx[j]];
+    }
+    if (chunk == 1) load_partials<EPT, 1, CMAX>(t, branch + src, idx, 0, n_partials, partial_stride);
+    else if (chunk == 2) load_partials<EPT, 2, CMAX>(t, branch + src, idx, 0, n_partials, partial_stride);
+    else if (chunk == 4) load_partials<EPT, 4, CMAX>(t, branch + src, idx, 0, n_partials, partial_stride);
+    else load_partials<EPT, CMAX, CMAX>(t, branch + src, idx, 0, n_partials, partial_stride);
+  }
+  // ---- arithmetic
+  float wq[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    xv[j] = in_row[j] ? xv[j] : 0.f;
+    wq[j] = (w_pre && in_row[j]) ? raw_to_f32(wq_raw[j]) : 0.f;
     bv[j] = 0.f;
   }
   if (branch) {
-    float wp[EPT];
+    // partial sums are added in their order, CMAX at a time
+    for (int p0 = 0; p0 < n_partials; p0 += CMAX) {
+      if (p0 > 0) load_partials<EPT, CMAX, CMAX>(t, branch + src, idx, p0, n_partials, partial_stride);
 #pragma unroll
-    for (int j = 0; j < EPT; ++j) {
-      const int i = threadIdx.x + j * blockDim.x;
-      wp[j] = (w_post && i < H) ? load_f32(w_post, i) : 0.f;
-      if (i < H) {
-        // partial sums are added in their order; eight loads are in flight at a time
-        float v = 0.f;
-        for (int p0 = 0; p0 < n_partials; p0 += 8) {
-          float t[8];
+      for (int j = 0; j < EPT; ++j)
 #pragma unroll
-          for (int p = 0; p < 8; ++p) t[p] = (p0 + p < n_partials) ? branch[src + i + (size_t)(p0 + p) * partial_stride] : 0.f;
-#pragma unroll
-          for (int p = 0; p < 8; ++p) v += t[p];
-        }
-        bv[j] = v;
-      }
+        for (int p = 0; p < CMAX; ++p)
+          if (p < chunk) bv[j] += (in_row[j] && p0 + p < n_partials) ? t[j][p] : 0.f;
     }
     if (w_post) {
       float ss = 0.f;
@@ -165,13 +206,12 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
       const float mean = ss / (float)H;
       const float inv_b = FULL ? 1.f / sqrtf(mean + eps_post) : rsqrtf(mean + eps_post);
 #pragma unroll
-      for (int j = 0; j < EPT; ++j) bv[j] = bv[j] * inv_b * (off_post + wp[j]);
+      for (int j = 0; j < EPT; ++j) bv[j] = bv[j] * inv_b * (off_post + (in_row[j] ? raw_to_f32(wp_raw[j]) : 0.f));
     }
 #pragma unroll
     for (int j = 0; j < EPT; ++j) {
-      const int i = threadIdx.x + j * blockDim.x;
       xv[j] += bv[j];
-      if (i < H) resid[src + i] = xv[j];
+      if (in_row[j]) resid[src + idx[j]] = xv[j];
     }
   }
   if (!out) return;
@@ -186,9 +226,104 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
     inv = FULL ? 1.f / sqrtf(mean + eps_pre) : rsqrtf(mean + eps_pre);
   }
 #pragma unroll
-  for (int j = 0; j < EPT; ++j) {
-    const int i = threadIdx.x + j * blockDim.x;
-    if (i < H) store_f32(o, out_index(out_layout, r, i, H), w_pre ? xv[j] * inv * (off_pre + wq[j]) : xv[j]);
+  for (int j = 0; j < EPT; ++j)
+    if (in_row[j]) store_f32(o, out_index(out_layout, r, idx[j], H), w_pre ? xv[j] * inv * (off_pre + wq[j]) : xv[j]);
+}
+
+// The same operation for many rows (prompts): one wave per row, four rows a block, four consecutive
+// elements a lane at a time (H a multiple of 4, at most 256 * K4).  No barriers: the sums go through the
+// wave's lanes.  Reduction orders differ from the block-per-row kernels by rounding only.
+template <typename TW> __device__ __forceinline__ float4 load4_f32(const TW* p, int e);
+template <> __device__ __forceinline__ float4 load4_f32<float>(const float* p, int e) { return *reinterpret_cast<const float4*>(p + e); }
+template <> __device__ __forceinline__ float4 load4_f32<bf16_t>(const bf16_t* p, int e) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p + e);
+  return float4{bf16_bits_to_f32(v.x & 0xffffu), bf16_bits_to_f32(v.x >> 16), bf16_bits_to_f32(v.y & 0xffffu), bf16_bits_to_f32(v.y >> 16)};
+}
+
+template <typename TW, typename TO, bool FULL, int K4>
+__global__ __launch_bounds__(256) void add_norm_rows_kernel(float* __restrict__ resid, const float* __restrict__ branch,
+                                                            int n_partials, size_t partial_stride,
+                                                            const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
+                                                            TO* __restrict__ out, int T, int H,
+                                                            float eps_post, float eps_pre, float off_post, float off_pre,
+                                                            int out_layout) {
+  const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= T) return;
+  const size_t src = (size_t)r * H;
+  int e[K4];
+  bool ok[K4];
+#pragma unroll
+  for (int k = 0; k < K4; ++k) {
+    const int i = (k * 64 + lane) * 4;
+    ok[k] = i < H;
+    e[k] = min(i, H - 4);                                    // clamped: loads are unconditional
+  }
+  const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4 xv[K4], bv[K4];
+#pragma unroll
+  for (int k = 0; k < K4; ++k) xv[k] = *reinterpret_cast<const float4*>(resid + src + e[k]);
+#pragma unroll
+  for (int k = 0; k < K4; ++k) bv[k] = zero4;
+  if (branch) {
+    for (int p = 0; p < n_partials; ++p) {                   // partial sums in their order
+      float4 t[K4];
+#pragma unroll
+      for (int k = 0; k < K4; ++k) t[k] = *reinterpret_cast<const float4*>(branch + (size_t)p * partial_stride + src + e[k]);
+#pragma unroll
+      for (int k = 0; k < K4; ++k) { bv[k].x += t[k].x; bv[k].y += t[k].y; bv[k].z += t[k].z; bv[k].w += t[k].w; }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < K4; ++k) {
+    if (!ok[k]) { xv[k] = zero4; bv[k] = zero4; }
+  }
+  if (branch) {
+    if (w_post) {
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < K4; ++k) ss += bv[k].x * bv[k].x + bv[k].y * bv[k].y + bv[k].z * bv[k].z + bv[k].w * bv[k].w;
+      ss = wave_sum(ss);
+      const float mean = ss / (float)H;
+      const float inv_b = FULL ? 1.f / sqrtf(mean + eps_post) : rsqrtf(mean + eps_post);
+#pragma unroll
+      for (int k = 0; k < K4; ++k) {
+        const float4 w = load4_f32<TW>(w_post, e[k]);
+        bv[k].x = bv[k].x * inv_b * (off_post + w.x);
+        bv[k].y = bv[k].y * inv_b * (off_post + w.y);
+        bv[k].z = bv[k].z * inv_b * (off_post + w.z);
+        bv[k].w = bv[k].w * inv_b * (off_post + w.w);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < K4; ++k) {
+      xv[k].x += bv[k].x; xv[k].y += bv[k].y; xv[k].z += bv[k].z; xv[k].w += bv[k].w;
+      if (ok[k]) *reinterpret_cast<float4*>(resid + src + e[k]) = xv[k];
+    }
+  }
+  if (!out) return;
+  float inv = 1.f;
+  if (w_pre) {
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < K4; ++k) ss += xv[k].x * xv[k].x + xv[k].y * xv[k].y + xv[k].z * xv[k].z + xv[k].w * xv[k].w;
+    ss = wave_sum(ss);
+    const float mean = ss / (float)H;
+    inv = FULL ? 1.f / sqrtf(mean + eps_pre) : rsqrtf(mean + eps_pre);
+  }
+#pragma unroll
+  for (int k = 0; k < K4; ++k) {
+    if (!ok[k]) continue;
+    float4 o = xv[k];
+    if (w_pre) {
+      const float4 w = load4_f32<TW>(w_pre, e[k]);
+      o = float4{xv[k].x * inv * (off_pre + w.x), xv[k].y * inv * (off_pre + w.y), xv[k].z * inv * (off_pre + w.z), xv[k].w * inv * (off_pre + w.w)};
+    }
+    const size_t at = out_index(out_layout, r, e[k], H);     // four consecutive elements are neighbours in both layouts
+    if constexpr (sizeof(TO) == 4) {
+      *reinterpret_cast<float4*>((float*)out + at) = o;
+    } else {
+      *reinterpret_cast<uint2*>((bf16_t*)out + at) = uint2{pack_bf16x2(o.x, o.y), pack_bf16x2(o.z, o.w)};
+    }
   }
 }
 
@@ -204,18 +339,28 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
   ALICE_CHECK(out_layout == 0 || (out_layout == 1 && out && out_dtype == DT_BF16 && H % 32 == 0),
               "add_norm: output in fragment order needs bfloat16 and a width that is a multiple of 32");
   if (T == 0) return 0;
-  // Rows up to 8192 wide are held in registers: 256 threads x 1..4 elements, then 1024 threads x 4 or 8.
+  // Rows up to 8192 wide are held in registers, 1 to 8 elements a thread; the block is just as wide as the
+  // row needs (a multiple of 64 threads), so that few threads are beyond its end.  Few rows: many threads
+  // with few elements each (the step waits for this kernel); many rows: fewer threads, more rows per CU.
   int threads = H >= 2048 ? 512 : 256, ept = 0;
-  if (H <= 1024) { threads = 256; ept = H <= 256 ? 1 : (H <= 512 ? 2 : 4); }
-  else if (H <= 4096) { threads = 1024; ept = 4; }
-  else if (H <= 8192) { threads = 1024; ept = 8; }
-  // Many rows: smaller blocks with more elements a thread keep more rows and more loads in flight on a CU.
-  if (T >= 256 && H > 1024 && H <= 4096) { threads = H <= 2048 ? 256 : 512; ept = 8; }
+  if (H <= 8192) {
+    ept = H <= 256 ? 1 : (H <= 512 ? 2 : (H <= 4096 ? 4 : 8));
+    threads = ceil_div(ceil_div(H, ept), 64) * 64;
+  }
 #define ARGS resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, \
              eps_post, eps_pre, off_post, off_pre, out_layout
+  // Many rows, no gather: a wave per row.
+  const bool aligned = (((uintptr_t)resid | (uintptr_t)branch | (uintptr_t)out | (uintptr_t)w_post | (uintptr_t)w_pre) & 15) == 0;
+  const int k4 = (!rows && aligned && T >= 128 && H % 4 == 0 && H >= 256 && H <= 4096 && (partial_stride % 4 == 0 || !branch)) ? ceil_div(H, 256) : 0;
+#define ROWS(TW, TO, FULL, K4) add_norm_rows_kernel<TW, TO, FULL, K4><<<ceil_div(T, 4), 256, 0, stream>>>(                \
+    resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, T, H, eps_post, eps_pre, \
+    off_post, off_pre, out_layout)
 #define LAUNCH(TW, TO, FULL)                                                                         \
   do {                                                                                               \
-    if (ept == 1) add_norm_regs_kernel<TW, TO, FULL, 1><<<T, threads, 0, stream>>>(ARGS);            \
+    if (k4 > 0 && k4 <= 4) ROWS(TW, TO, FULL, 4);                                                    \
+    else if (k4 > 4 && k4 <= 9) ROWS(TW, TO, FULL, 9);                                               \
+    else if (k4 > 9) ROWS(TW, TO, FULL, 16);                                                         \
+    else if (ept == 1) add_norm_regs_kernel<TW, TO, FULL, 1><<<T, threads, 0, stream>>>(ARGS);            \
     else if (ept == 2) add_norm_regs_kernel<TW, TO, FULL, 2><<<T, threads, 0, stream>>>(ARGS);       \
     else if (ept == 4) add_norm_regs_kernel<TW, TO, FULL, 4><<<T, threads, 0, stream>>>(ARGS);       \
     else if (ept == 8) add_norm_regs_kernel<TW, TO, FULL, 8><<<T, threads, 0, stream>>>(ARGS);       \
@@ -225,6 +370,7 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
     if (full_precision) LAUNCH(TW, TO, true); else LAUNCH(TW, TO, false);
   }));
 #undef LAUNCH
+#undef ROWS
 #undef ARGS
   ALICE_LAUNCH_CHECK();
   return 0;

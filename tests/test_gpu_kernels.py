@@ -70,6 +70,40 @@ def test_add_norm_all_forms(wdt, odt, full, H):
     close(out3, P.rms_norm(x0.double()[rows.long()], wq.double(), 1e-5), tol, tol)
 
 
+@pytest.mark.parametrize("H", [256, 1000, 2304, 4096])
+@pytest.mark.parametrize("S", [1, 3])
+@pytest.mark.parametrize("odt", ["float32", "bfloat16"])
+def test_add_norm_many_rows(H, S, odt):
+    # prompts take another kernel (a wave per row) than single tokens do
+    T = 300
+    x0 = rnd(T, H, seed=2, scale=3.0)
+    br = rnd(S, T, H, seed=3, scale=0.5) if S > 1 else rnd(T, H, seed=3, scale=0.5)
+    wp, wq = rnd(H, seed=4, scale=0.1, dtype=torch.bfloat16), rnd(H, seed=5, scale=0.1, dtype=torch.bfloat16)
+    tol = 2e-6 if odt == "float32" else 2 ** -8
+    x = x0.clone()
+    out = torch.full((T, H), float("nan"), dtype=DT[odt], device=DEV)
+    ops.add_norm(x, br, wp, wq, out, eps_post=1e-6, eps_pre=1e-5, off_post=1.0, off_pre=1.0, n_partials=S, full_precision=False)
+    b = br.double().sum(0) if S > 1 else br.double()
+    xr = x0.double() + P.rms_norm(b, wp.double(), 1e-6)
+    close(x, xr, 1e-5)
+    close(out, P.rms_norm(xr, wq.double(), 1e-5), tol * 4, tol)
+    # the single-token kernel on the same rows: equal up to the order of the sums
+    x2, out2 = x0[:7].clone(), torch.empty(7, H, dtype=DT[odt], device=DEV)
+    ops.add_norm(x2, br[:, :7].contiguous() if S > 1 else br[:7].contiguous(), wp, wq, out2, eps_post=1e-6, eps_pre=1e-5,
+                 off_post=1.0, off_pre=1.0, n_partials=S, full_precision=False)
+    close(x[:7], x2, 2e-6, 1e-6)
+    # add only, and norm only
+    x = x0.clone()
+    ops.add_norm(x, br, None, None, None, n_partials=S, full_precision=False)
+    close(x, x0.double() + b, 1e-5)
+    ops.add_norm(x0, None, None, wq, out, eps_pre=1e-5, off_pre=0.0, full_precision=False)
+    close(out, P.rms_norm(x0.double(), wq.double() - 1.0, 1e-5), tol * 4, tol)
+    if H % 32 == 0 and odt == "bfloat16":
+        flat = torch.empty((-(-T // 16) * 16) * H, dtype=torch.bfloat16, device=DEV)
+        ops.add_norm(x0, None, None, wq, flat, eps_pre=1e-5, off_pre=0.0, full_precision=False, out_layout=ops.LAYOUT_FRAG16)
+        assert torch.equal(acts_from_fragments(flat, T, H), out.cpu())
+
+
 def test_rms_norm_reference_vector_on_device():
     x = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)                       # llama3.rs:20482-20498
     out = torch.empty_like(x)
