@@ -324,6 +324,153 @@ def test_toy_architecture_against_its_plain_replica():
     assert (got.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
 
 
+# ------------------------------------------------------------------ a second toy: routing and another position encoding
+class ToyRoutedFF(Part):
+    """A feed-forward with routing: router logits in 32-bit, the two best of E experts per token, their
+    softmax weights, experts y = relu(x W1_e^T) W2_e^T.  In torch: a test of the interface (a feed-forward sees
+    x and the step's context, nothing else), not a kernel."""
+
+    def __init__(self, precision, *, hidden_size, inner, experts):
+        self.H, self.I, self.E = hidden_size, inner, experts
+        self.w = {}
+
+    def param_specs(self):
+        specs = {"router.weight": ParamSpec((self.E, self.H), 0.5)}
+        for e in range(self.E):
+            specs[f"experts.{e}.up.weight"] = ParamSpec((self.I, self.H), 0.1)
+            specs[f"experts.{e}.down.weight"] = ParamSpec((self.H, self.I), 0.1)
+        return specs
+
+    def assign(self, name, t):
+        self.w[name] = t.float()
+
+    @staticmethod
+    def route(x, w, E, I, H, dtype):
+        logits = x.to(dtype) @ w["router.weight"].to(dtype).T
+        top, idx = logits.topk(2, dim=-1)
+        gate = torch.softmax(top, dim=-1)
+        out = torch.zeros(x.shape[0], H, dtype=dtype, device=x.device)
+        for e in range(E):
+            for slot in range(2):
+                rows = (idx[:, slot] == e).nonzero().flatten()
+                if rows.numel():
+                    h = torch.relu(x[rows].to(dtype) @ w[f"experts.{e}.up.weight"].to(dtype).T)
+                    out[rows] += gate[rows, slot, None] * (h @ w[f"experts.{e}.down.weight"].to(dtype).T)
+        return out, idx
+
+    def forward(self, x, ctx):
+        out, self.last_choice = self.route(x, self.w, self.E, self.I, self.H, torch.float32)
+        return out.contiguous()
+
+
+class ToyInterleavedRotation(Part):
+    """Another position encoding: rotation of the pairs (2j, 2j + 1) (the reference's other pairing,
+    llama3.rs:5323-5336), done in torch; keys and values then go into the cache through the library's write
+    without rotation.  What a position encoding owes the attention mixer is rotate_and_store, nothing more."""
+
+    def __init__(self, precision, device, *, dim, theta, max_positions):
+        j = torch.arange(dim // 2, dtype=torch.float64)
+        ang = torch.arange(max_positions, dtype=torch.float64)[:, None] * theta ** (-2.0 * j / dim)
+        self.cos, self.sin = torch.cos(ang).float().to(device), torch.sin(ang).float().to(device)
+        self.none = POSITIONS.get("none")(precision, device)
+
+    def rotate(self, x, positions):            # x: [T, heads, d]
+        c, s = self.cos[positions.long()][:, None, :].to(x.dtype), self.sin[positions.long()][:, None, :].to(x.dtype)
+        a, b = x[..., 0::2], x[..., 1::2]
+        return torch.stack([a * c - b * s, a * s + b * c], dim=-1).flatten(-2)
+
+    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim, kv_layout=0):
+        T = qkv.shape[0]
+        nq, nk = num_heads * head_dim, num_kv_heads * head_dim
+        rot = qkv.clone()
+        rot[:, :nq] = self.rotate(qkv[:, :nq].float().view(T, num_heads, head_dim), ctx.positions).reshape(T, nq).to(qkv.dtype)
+        rot[:, nq:nq + nk] = self.rotate(qkv[:, nq:nq + nk].float().view(T, num_kv_heads, head_dim), ctx.positions).reshape(T, nk).to(qkv.dtype)
+        self.none.rotate_and_store(rot, q_out, ctx, cache, num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
+                                   kv_layout=kv_layout)
+
+
+class ToyRoutedConfig(ToyConfig):
+    def plan(self):
+        H, V = self.d["width"], self.d["vocab"]
+        norm = lambda name: PartSpec("rmsnorm", {"dim": H, "eps": 1e-5, "weight_offset": 0.0}, name)
+        att = lambda: PartSpec("attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 3, "head_dim": 16, "scale": 0.25,
+                                             "position": "twist"}, "attn")
+        ffs = [PartSpec("toy_routed", {"hidden_size": H, "inner": 40, "experts": 3}, "moe"), PartSpec("toy_mlp", {"hidden_size": H}, "ff")]
+        layers = [LayerPlan(block="prenorm", mixer=att(), feed_forward=ffs[i % 2], norms={"pre_mixer": norm("n1"), "pre_ff": norm("n2")},
+                            prefix=f"blocks.{i}.") for i in range(self.d["depth"])]
+        return ModelPlan(vocab_size=V, hidden_size=H, max_positions=128,
+                         embedding=PartSpec("embedding", {"vocab_size": V, "dim": H, "scale": 1.0}, "emb"),
+                         positions={"twist": PartSpec("toy_interleaved", {"dim": 16, "theta": 50.0, "max_positions": 128})},
+                         layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(self.d["depth"])),
+                         final_norm=norm("final"), head=PartSpec("lm_head", {"vocab_size": V, "dim": H, "tied_to": "emb"}, "head"))
+
+
+def toy_routed_plain(model, tokens):
+    lm = model.lm
+    E = lm.embedding.table.weight.double().cpu()
+    x = E[torch.tensor(tokens)]
+    T = len(tokens)
+    rms = lambda v, n: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + n.eps) * (n.weight_offset + n.weight.double().cpu())
+    pos = torch.arange(T)
+    ang = pos.double()[:, None] * 50.0 ** (-2.0 * torch.arange(8, dtype=D) / 16)
+    def twist(v):        # [T, heads, 16], pairs (2j, 2j+1)
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        a, b = v[..., 0::2], v[..., 1::2]
+        return torch.stack([a * c - b * s, a * s + b * c], dim=-1).flatten(-2)
+    choices = []
+    for layer in lm.layers:
+        h = rms(x, layer.norms["pre_mixer"])
+        W = layer.mixer.qkv.weight.double().cpu()
+        q, k, v = (h @ W[:48].T).view(T, 3, 16), (h @ W[48:96].T).view(T, 3, 16), (h @ W[96:].T).view(T, 3, 16)
+        o = P.attention_core(twist(q), twist(k), v, 0.25, None, None)
+        x = x + o.reshape(T, 48) @ layer.mixer.o.weight.double().cpu().T
+        h = rms(x, layer.norms["pre_ff"])
+        ff = layer.feed_forward
+        if isinstance(ff, ToyRoutedFF):
+            y, idx = ToyRoutedFF.route(h, {k_: v_.cpu() for k_, v_ in ff.w.items()}, ff.E, ff.I, ff.H, D)
+            choices.append(idx)
+            x = x + y
+        else:
+            x = x + torch.relu(h @ ff.w.double().cpu().T)
+    return rms(x, lm.final_norm) @ E.T, choices
+
+
+def test_toy_architecture_with_routing_and_another_position_encoding():
+    FEED_FORWARDS.register("toy_mlp", ToyMLP)
+    FEED_FORWARDS.register("toy_routed", ToyRoutedFF)
+    POSITIONS.register("toy_interleaved", ToyInterleavedRotation)
+    alice.register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig)
+    raw = {"architectures": ["ToyRoutedForCausalLM"], "width": 48, "vocab": 61, "depth": 3}
+    model = alice.Model.random(raw, seed=5, dtype="float32", stored_dtype=torch.float32)
+    assert "blocks.0.moe.experts.2.down.weight" in model.lm.param_specs() and "blocks.1.ff.w.weight" in model.lm.param_specs()
+    eng = model.engine(max_tokens=256, max_seqs=2)
+    seqs = [[5, 9, 3, 60, 1, 22, 8, 8, 41, 2, 13, 0, 33, 17], [7, 7, 30, 12, 55]]
+    slots = eng.open(2)
+    whole = eng.step(slots, seqs, "all")
+    eng.close(slots)
+    refs = [toy_routed_plain(model, t) for t in seqs]
+    ref = torch.cat([r[0] for r in refs])
+    assert (whole.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
+    # the routing really spreads tokens over the experts (else the test would not see a wrong choice)
+    assert len(set(torch.cat([c.flatten() for c in refs[0][1]]).tolist())) == 3
+    # cut into steps, in a batch whose shorter request ends earlier: the same logits
+    slots = eng.open(2)
+    first = eng.step(slots, [s[:3] for s in seqs], "all")
+    outs = {0: [first[:3]], 1: [first[3:]]}
+    for i in range(3, len(seqs[0])):
+        live = [b for b in (0, 1) if i < len(seqs[b])]
+        lg = eng.step([slots[b] for b in live], [[seqs[b][i]] for b in live], "last")
+        for row, b in enumerate(live):
+            outs[b].append(lg[row:row + 1])
+        if i + 1 == len(seqs[1]):
+            eng.close([slots[1]])
+    eng.close([slots[0]])
+    cut = torch.cat([torch.cat(outs[0]), torch.cat(outs[1])])
+    assert (cut - whole).abs().max() < 1e-5
+    eng.cache.check_consistent()
+
+
+
 @pytest.mark.parametrize("prec", PRECS)
 def test_embedding_and_tied_head_parts(prec):
     from alice_llm_amd.parts import EMBEDDINGS, HEADS
