@@ -194,24 +194,39 @@ class Cache:
         """Make room for n_new[i] more tokens in slots[i]; raises before anything changes."""
         if len(set(slots)) != len(slots):
             raise CacheError(f"a step names a slot twice: {list(slots)}")
-        new_lens = [self.slots.length(s) + n for s, n in zip(slots, n_new)]
+        lens = [self.slots.length(s) for s in slots]
+        if max(n_new) == 1 and min(n_new) == 1:
+            # one token each: only a sequence whose length is a multiple of the page size needs a page
+            P = self.page_size
+            pairs = [(s, l + 1) for s, l in zip(slots, lens) if l % P == 0]
+            if not pairs:
+                return
+        else:
+            pairs = [(s, l + n) for s, l, n in zip(slots, lens, n_new)]
         for g in self.groups:
-            need = sum(g.pages_needed(s, l) for s, l in zip(slots, new_lens))
+            need = sum(g.pages_needed(s, l) for s, l in pairs)
             if need > g.n_free():
                 raise CacheError(
                     f"the cache is full: this step needs {need} more pages of {self.page_size} tokens in the group of "
                     f"layers {g.layers}, {g.n_free()} are free (cache sized for {self.max_tokens} tokens)")
         for g in self.groups:
-            for s, l in zip(slots, new_lens):
+            for s, l in pairs:
                 if g.pages_needed(s, l):
                     self.version += 1
                 g.grow(s, l)
 
     def commit(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
+        P = self.page_size
         for s, n in zip(slots, n_new):
             self.slots.advance(s, n)
+            length = self.slots.length(s)
             for g in self.groups:
-                if g.trim(s, self.slots.length(s)):
+                w = g.need.window
+                # a page of a windowed group can only fall out of reach when the oldest key that the next
+                # query needs has just moved onto a new page (one token) or moved at all (several)
+                if w is None or length + 1 - w <= 0 or (n == 1 and (length + 1 - w) % P != 0):
+                    continue
+                if g.trim(s, length):
                     self.version += 1
 
     def block_table_rows(self, group: int, slots: Sequence[int], width: int) -> List[List[int]]:

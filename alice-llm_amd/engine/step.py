@@ -13,6 +13,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from ..cache import Cache, CacheError
@@ -101,8 +102,15 @@ class _DecodeGraph:
         for n in sizes:
             self.offs.append(self.offs[-1] + n)
         self.static = torch.zeros(self.offs[-1], dtype=torch.int32, device=dev)
+        # The step's integers are kept in a host array that is updated in place (the block tables only when they
+        # change) and copied through one of four pinned buffers; a pinned buffer is written again only after the
+        # copy that last read it has run.  numpy views: a step writes a handful of short slices, and the time this
+        # takes is time the GPU waits between two steps.
+        self.shadow = np.zeros(self.offs[-1], dtype=np.int32)
         self.staging = [torch.zeros(self.offs[-1], dtype=torch.int32).pin_memory() for _ in range(4)]
-        self.events = [None] * 4
+        self.staging_np = [t.numpy() for t in self.staging]
+        self.events = [torch.cuda.Event() for _ in range(4)]
+        self.used = [False] * 4
         self.turn = 0
         part = lambda i: self.static[self.offs[i]:self.offs[i + 1]]
         self.block_tables = [part(7 + g).view(B, self.width) for g in range(n_groups)]
@@ -111,6 +119,10 @@ class _DecodeGraph:
                                max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
                                start_lens=[0] * B, slot_ids=[0] * B,
                                fragment_activations=engine.model.precision.act == torch.bfloat16 and B <= 64)
+        o = self.offs
+        self.shadow[o[2]:o[3]] = np.arange(B)                # constant parts
+        self.shadow[o[4]:o[5]] = np.arange(B)
+        self.shadow[o[5]:o[6]] = np.arange(B + 1)
         self.graph = None
         self.logits = None
         self.tables_version = None
@@ -119,35 +131,29 @@ class _DecodeGraph:
     def fill(self, engine: "Engine", slots, tokens, start) -> None:
         """Write this step's integers into a pinned buffer and queue its copy to the device."""
         B, n = self.batch, len(slots)
-        i = self.turn = (self.turn + 1) % len(self.staging)
-        if self.events[i] is not None:
-            self.events[i].synchronize()                     # the copy that last used this buffer has run
-        hp = self.staging[i]
-        o = self.offs
-        prev = self.staging[(i - 1) % len(self.staging)]
-        same_tables = (self.tables_version == engine.cache.version and self.tables_slots == list(slots))
-        if same_tables:
-            hp[o[7]:].copy_(prev[o[7]:])
-        else:
+        o, sh = self.offs, self.shadow
+        if self.tables_version != engine.cache.version or self.tables_slots != list(slots):
             for g in range(len(self.block_tables)):
                 rows = engine.cache.block_table_rows(g, slots, self.width)
-                flat = [p for r in rows for p in r] + [0] * ((B - n) * self.width)
-                hp[o[7 + g]:o[8 + g]] = torch.tensor(flat, dtype=torch.int32)
+                tab = sh[o[7 + g]:o[8 + g]].reshape(B, self.width)
+                tab[:n] = rows
+                tab[n:] = 0                                  # padded rows: the spare page
             self.tables_version, self.tables_slots = engine.cache.version, list(slots)
-        pad = B - n
-        hp[o[0]:o[1]] = torch.tensor(list(tokens) + [0] * pad, dtype=torch.int32)
-        hp[o[1]:o[2]] = torch.tensor(list(start) + [0] * pad, dtype=torch.int32)
-        hp[o[6]:o[7]] = torch.tensor([l + 1 for l in start] + [1] * pad, dtype=torch.int32)
-        if self.graph is None:                               # constant parts, written once per buffer set
-            for buf in self.staging:
-                buf[o[2]:o[3]] = torch.arange(B, dtype=torch.int32)
-                buf[o[3]:o[4]] = 0
-                buf[o[4]:o[5]] = torch.arange(B, dtype=torch.int32)
-                buf[o[5]:o[6]] = torch.arange(B + 1, dtype=torch.int32)
-        self.static.copy_(hp, non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record()
-        self.events[i] = ev
+        sh[o[0]:o[0] + n] = tokens
+        sh[o[0] + n:o[1]] = 0
+        sh[o[1]:o[1] + n] = start
+        sh[o[1] + n:o[2]] = 0
+        ctx_lens = sh[o[6]:o[7]]
+        ctx_lens[:n] = start
+        ctx_lens[:n] += 1
+        ctx_lens[n:] = 1
+        i = self.turn = (self.turn + 1) % len(self.staging)
+        if self.used[i]:
+            self.events[i].synchronize()                     # the copy that last used this buffer has run
+        np.copyto(self.staging_np[i], sh)
+        self.static.copy_(self.staging[i], non_blocking=True)
+        self.events[i].record()
+        self.used[i] = True
 
 
 class Engine:
