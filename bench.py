@@ -146,7 +146,9 @@ def main() -> int:
         print(f"[bench] decode_b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s @ batch 8, Gemma-2-2B bf16 (points: batch 1/64; prefill tok/s @ 2,048 tok)",
+        "metric": (f"decode tok/s @ batch {args.batch}, Gemma-2-{args.preset.upper()} {short} "
+                   f"(points: batch {'/'.join(str(int(x)) for x in args.points.split(',') if x) or '-'}; "
+                   f"prefill tok/s @ {args.prompt:,} tok)"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
