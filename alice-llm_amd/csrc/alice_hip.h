@@ -4,11 +4,12 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 1
+#define ALICE_ABI_VERSION 2
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
 #define ALICE_EPI_SOFTCAP 2   // y = cap * tanh(y / cap)
+#define ALICE_EPI_ROPE 3      // internal: rotation and cache write (alice_linear_rope_cache)
 
 #define ALICE_LAYOUT_ROW 0     // row-major [N, K]
 #define ALICE_LAYOUT_FRAG16 1  // bfloat16 in 16x32 MFMA fragments, see linear_mfma.hip
@@ -61,7 +62,16 @@ int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool
                            const float* cos_t, const float* sin_t, const int* positions,
                            const int* seq_of_token, const int* block_table, int bt_stride, int T,
                            int row_width, int nH, int nKV, int d, int rotary_dim, int page_size, int n_pages,
-                           int kv_layout, hipStream_t stream);
+                           int kv_layout, int interleaved, hipStream_t stream);
+
+// The fused q|k|v projection of single tokens (at most 64), with the rotation and the cache write as its
+// epilogue: x [M, K] (row-major or fragment order), W in the fragment layout with the rows of every q and k
+// head in pair order (rows j and j + d/2 of a head at 2j and 2j + 1).  Writes what alice_linear followed by
+// alice_rope_cache_write (interleaved) would: q_out [M, nH * d] and the token's keys and values in the cache.
+int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, int K, void* q_out, void* k_pool,
+                            void* v_pool, const float* cos_t, const float* sin_t, const int* positions,
+                            const int* seq_of_token, const int* block_table, int bt_stride, int nH, int nKV, int d,
+                            int page_size, int n_pages, int kv_layout, hipStream_t stream);
 
 int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
                             const int* positions, const int* seq_of_token, const int* block_table,

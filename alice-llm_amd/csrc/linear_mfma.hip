@@ -17,6 +17,7 @@
 // GeGLU (llama3.rs:14519-14534) and softcap (llama3.rs:14606-14611) epilogues.
 #include "common.h"
 #include "alice_hip.h"
+#include "kv_layout.h"
 
 namespace {
 
@@ -85,6 +86,19 @@ __device__ __forceinline__ void store4_frag(bf16_t* __restrict__ y, int m, int n
   *reinterpret_cast<uint2*>(y + off) = pk;
 }
 
+// What the rotation epilogue needs: where q goes, the cache, the tables and the geometry.
+struct RopeArgs {
+  bf16_t* q_out;
+  bf16_t* k_pool;
+  bf16_t* v_pool;
+  const float* cos_t;
+  const float* sin_t;
+  const int* positions;
+  const int* seq_of_token;
+  const int* block_table;
+  int bt_stride, nH, nKV, d, page_size, n_pages, layout;
+};
+
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
 // Block: NW waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + NW, ...; the parts of
 // waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
@@ -98,7 +112,7 @@ __device__ __forceinline__ void store4_frag(bf16_t* __restrict__ y, int m, int n
 template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                            int kt_per_slice, float epi, int y_frag) {
+                                                            int kt_per_slice, float epi, int y_frag, RopeArgs ra) {
   extern __shared__ __align__(16) float red[];            // [NW - 1][RT*MT][64][4]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -208,6 +222,53 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
         acc[i][j] += p;
       }
 
+  if constexpr (EPI == ALICE_EPI_ROPE) {
+    // The rows of W are all q heads, all k heads, all v heads, the rows of every q and k head in pair order:
+    // this lane's four features of a tile are two whole rotated pairs (or four elements of a value head).
+    // The sums are rounded to bfloat16 before the rotation, as they are when the projection and the
+    // rotation are separate kernels: both ways give the same bits.
+    const int d = ra.d, half = d >> 1;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      if (!row_ok[j]) continue;
+      const int m = row[j];
+      const int pos = ra.positions[m];
+      const int tp = pos % ra.page_size;
+      const int page = ra.block_table[(size_t)ra.seq_of_token[m] * ra.bt_stride + pos / ra.page_size];
+      const bool page_ok = page >= 0 && page < ra.n_pages;
+      const size_t page_base = (size_t)(page_ok ? page : 0) * ra.nKV * ra.page_size * d;
+#pragma unroll
+      for (int i = 0; i < RT; ++i) {
+        if (tile[i] >= NT) continue;
+        const int n = tile[i] * 16 + g * 4;                // first of this lane's four features, in W's row order
+        const int head = n / d, w = n % d;
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[i][j][e]);
+        if (head < ra.nH + ra.nKV) {
+          const int p0 = w >> 1;                           // the pairs p0 and p0 + 1 of the head
+          const float2 c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)pos * half + p0);
+          const float2 sn = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)pos * half + p0);
+          const uint32_t lo = pack_bf16x2(x[0] * c.x - x[1] * sn.x, x[2] * c.y - x[3] * sn.y);
+          const uint32_t hi = pack_bf16x2(x[0] * sn.x + x[1] * c.x, x[2] * sn.y + x[3] * c.y);
+          if (head < ra.nH) {
+            bf16_t* dst = ra.q_out + ((size_t)m * ra.nH + head) * d;
+            *reinterpret_cast<uint32_t*>(dst + p0) = lo;
+            *reinterpret_cast<uint32_t*>(dst + p0 + half) = hi;
+          } else if (page_ok) {
+            bf16_t* dst = ra.k_pool + page_base + (size_t)(head - ra.nH) * ra.page_size * d;
+            *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, tp, p0, d)) = lo;
+            *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, tp, p0 + half, d)) = hi;
+          }
+        } else if (page_ok) {
+          bf16_t* dst = ra.v_pool + page_base + (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[v_offset(ra.layout, tp, w + e, d)] = f32_to_bf16(x[e]);
+        }
+      }
+    }
+    return;
+  }
   TO* yo = y + (size_t)blockIdx.y * M * N;                // the slice's partial sum
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
@@ -419,7 +480,7 @@ __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restr
 
 template <int RT, int MT, int EPI, typename TO>
 int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
-                  hipStream_t s) {
+                  hipStream_t s, const RopeArgs& ra = RopeArgs{}) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int groups = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, RT / 2) : ceil_div(NT, RT);
   const int per = ceil_div(KT, split);
@@ -429,12 +490,12 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   const bool eight = (RT * MT <= 4) && per >= 32 && groups * split < 2048;
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
-    if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
-    else linear_skinny_kernel<RT, MT, 8, EPI, TO, false, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
+    if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    else linear_skinny_kernel<RT, MT, 8, EPI, TO, false, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
   } else {
     const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-    if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
-    else linear_skinny_kernel<RT, MT, 4, EPI, TO, false, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag);
+    if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    else linear_skinny_kernel<RT, MT, 4, EPI, TO, false, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
   }
   ALICE_LAUNCH_CHECK();
   return 0;
@@ -584,4 +645,39 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
   BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
 #undef BY_EPI
+}
+
+extern "C" int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, int K, void* q_out, void* k_pool,
+                                       void* v_pool, const float* cos_t, const float* sin_t, const int* positions,
+                                       const int* seq_of_token, const int* block_table, int bt_stride, int nH, int nKV,
+                                       int d, int page_size, int n_pages, int kv_layout, hipStream_t stream) {
+  ALICE_CHECK(M >= 0 && M <= 64, "linear+rope: at most 64 tokens, found %d", M);
+  ALICE_CHECK(K > 0 && K % 8 == 0, "linear+rope: K must be a multiple of 8, found %d", K);
+  ALICE_CHECK(nH >= 1 && nKV >= 1 && d >= 16 && d % 16 == 0, "linear+rope: bad heads nH=%d nKV=%d d=%d (d must be a multiple of 16)", nH, nKV, d);
+  ALICE_CHECK(x && w && q_out && k_pool && v_pool && cos_t && sin_t && positions && seq_of_token && block_table,
+              "linear+rope: a pointer is missing");
+  ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)q_out & 3) == 0 && ((uintptr_t)cos_t & 7) == 0 &&
+              ((uintptr_t)sin_t & 7) == 0 && ((uintptr_t)k_pool & 3) == 0, "linear+rope: operands are not aligned");
+  ALICE_CHECK(x_layout == ALICE_LAYOUT_ROW || (x_layout == ALICE_LAYOUT_FRAG16 && K % 32 == 0),
+              "linear+rope: activations in fragment order need K %% 32 == 0, found K=%d", K);
+  ALICE_CHECK(page_size > 0 && n_pages > 0 && bt_stride > 0, "linear+rope: bad page geometry");
+  ALICE_CHECK(kv_layout == 0 || (kv_layout == 1 && page_size == 64 && d % 32 == 0),
+              "linear+rope: the fragment cache layout needs pages of 64 and head_dim %% 32 == 0");
+  if (M == 0) return 0;
+  const int N = (nH + 2 * nKV) * d;
+  RopeArgs ra{(bf16_t*)q_out, (bf16_t*)k_pool, (bf16_t*)v_pool, cos_t, sin_t, positions, seq_of_token, block_table,
+              bt_stride, nH, nKV, d, page_size, n_pages, kv_layout};
+  const int x_frag = x_layout == ALICE_LAYOUT_FRAG16;
+  const int rt = skinny_row_tiles(M, N, ALICE_EPI_NONE, 1, K);
+#define GO(RT, MT) return launch_skinny<RT, MT, ALICE_EPI_ROPE, bf16_t>(x, w, nullptr, M, N, K, 1, 0.f, x_frag, 0, stream, ra)
+#define BY_RT(MT)                \
+  do {                           \
+    if (rt >= 2) GO(2, MT);      \
+    GO(1, MT);                   \
+  } while (0)
+  if (M <= 16) BY_RT(1);
+  if (M <= 32) BY_RT(2);
+  BY_RT(4);
+#undef BY_RT
+#undef GO
 }

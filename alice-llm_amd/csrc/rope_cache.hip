@@ -6,21 +6,11 @@
 // v as it is (llama3.rs:14307-14331).  Dimensions at or beyond R pass through unchanged.
 #include "common.h"
 #include "alice_hip.h"
+#include "kv_layout.h"
 
-// Offsets of element e of the token at place t of a 64-position page of one kv head.  Layout 0 is
-// row-major [position][d]; layout 1 is the fragment layout that the matrix-core attention kernels
-// read (see attention_mfma.hip): keys in 16-position x 32-dim tiles, values in 32-position x 16-dim
-// tiles with the positions in the order the score tiles come out of the MFMA.
-__device__ __forceinline__ size_t k_offset(int layout, int t, int e, int d) {
-  if (layout == 0) return (size_t)t * d + e;
-  return ((size_t)((t >> 4) * (d >> 5) + (e >> 5)) * 64 + ((e & 31) >> 3) * 16 + (t & 15)) * 8 + (e & 7);
-}
-__device__ __forceinline__ size_t v_offset(int layout, int t, int e, int d) {
-  if (layout == 0) return (size_t)t * d + e;
-  const int tt = t & 31, w = tt & 15;
-  return ((size_t)((t >> 5) * (d >> 4) + (e >> 4)) * 64 + (w >> 2) * 16 + (e & 15)) * 8 + ((tt >> 4) * 4 + (w & 3));
-}
-
+// `interleaved`: the q and k heads of the qkv row come with the two elements of each rotated pair next to
+// each other, (j, j + R/2) at 2j and 2j + 1 (the order in which a projection whose rows were permuted that
+// way delivers them; only with R == d); the outputs are in the plain order either way.
 // One block per token.  qkv row of row_w elements: [nH*d | nKV*d | nKV*d | ...]; with no pools
 // only the q part is read.  cos/sin: [max_pos, R/2].
 // Cache pools: [page][nKV][page_size][d]; the page of position p of sequence s is
@@ -31,7 +21,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                   const int* __restrict__ block_table, int bt_stride, int row_w,
-                                  int nH, int nKV, int d, int R, int page_size, int n_pages, int layout) {
+                                  int nH, int nKV, int d, int R, int page_size, int n_pages, int layout, int interleaved) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = R >> 1;
@@ -63,7 +53,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
     for (int j = threadIdx.x; j < hd2; j += blockDim.x) {
       // the rotated pair (j, j + half) if j < half; elements at or beyond R pass through, spread over the items
       if (j < half) {
-        float x0 = load_f32(src, j), x1 = load_f32(src, j + half);
+        float x0 = load_f32(src, interleaved ? 2 * j : j), x1 = load_f32(src, interleaved ? 2 * j + 1 : j + half);
         float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
         store_f32(dst, at(j), x0 * c - x1 * s);
         store_f32(dst, at(j + half), x0 * s + x1 * c);
@@ -87,7 +77,7 @@ __global__ void rope_cache_vec_kernel(const bf16_t* __restrict__ qkv, bf16_t* __
                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                       const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                       const int* __restrict__ block_table, int bt_stride, int row_w,
-                                      int nH, int nKV, int d, int page_size, int n_pages, int layout) {
+                                      int nH, int nKV, int d, int page_size, int n_pages, int layout, int interleaved) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = d >> 1;
@@ -114,7 +104,16 @@ __global__ void rope_cache_vec_kernel(const bf16_t* __restrict__ qkv, bf16_t* __
     if (it < rot_items) {
       const int h = it / per_head, j = (it % per_head) * 8;
       const bf16_t* src = row + (size_t)h * d;
-      const uint4 lo = *reinterpret_cast<const uint4*>(src + j), hi = *reinterpret_cast<const uint4*>(src + j + half);
+      uint4 lo, hi;
+      if (interleaved) {
+        // pairs j .. j+7 lie at 2j .. 2j+15: even places are the first elements, odd places the second
+        const uint4 a = *reinterpret_cast<const uint4*>(src + 2 * j), b = *reinterpret_cast<const uint4*>(src + 2 * j + 8);
+        lo = uint4{(a.x & 0xffffu) | (a.y << 16), (a.z & 0xffffu) | (a.w << 16), (b.x & 0xffffu) | (b.y << 16), (b.z & 0xffffu) | (b.w << 16)};
+        hi = uint4{(a.x >> 16) | (a.y & 0xffff0000u), (a.z >> 16) | (a.w & 0xffff0000u), (b.x >> 16) | (b.y & 0xffff0000u), (b.z >> 16) | (b.w & 0xffff0000u)};
+      } else {
+        lo = *reinterpret_cast<const uint4*>(src + j);
+        hi = *reinterpret_cast<const uint4*>(src + j + half);
+      }
       const float4 c0 = *reinterpret_cast<const float4*>(cs + j), c1 = *reinterpret_cast<const float4*>(cs + j + 4);
       const float4 s0 = *reinterpret_cast<const float4*>(sn + j), s1 = *reinterpret_cast<const float4*>(sn + j + 4);
       const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
@@ -165,8 +164,9 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
                                       const float* cos_t, const float* sin_t, const int* positions,
                                       const int* seq_of_token, const int* block_table, int bt_stride,
                                       int T, int row_width, int nH, int nKV, int d, int rotary_dim, int page_size,
-                                      int n_pages, int kv_layout, hipStream_t stream) {
+                                      int n_pages, int kv_layout, int interleaved, hipStream_t stream) {
   ALICE_CHECK(dtype_ok(dtype), "rope: unknown dtype %d", dtype);
+  ALICE_CHECK(!interleaved || (rotary_dim == d && cos_t != nullptr), "rope: interleaved pairs need the whole head rotated");
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 2 && d % 2 == 0, "rope: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
   ALICE_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0, "rope: rotated width %d must be even and at most head_dim %d", rotary_dim, d);
   ALICE_CHECK((cos_t == nullptr) == (sin_t == nullptr), "rope: cos and sin tables must come together");
@@ -186,13 +186,13 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
     const int items = (nH + nKV) * (d / 16) + nKV * (d / 8);
     const int threads = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
     rope_cache_vec_kernel<<<T, threads, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_pool, (bf16_t*)v_pool,
-        cos_t, sin_t, positions, seq_of_token, block_table, bt_stride, row_width, nH, nKV, d, page_size, n_pages, kv_layout);
+        cos_t, sin_t, positions, seq_of_token, block_table, bt_stride, row_width, nH, nKV, d, page_size, n_pages, kv_layout, interleaved);
     ALICE_LAUNCH_CHECK();
     return 0;
   }
   DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<dim3(T, nH + (k_pool ? 2 * nKV : 0)), d >= 256 ? 128 : 64, 0, stream>>>(
       (const TT*)qkv, (TT*)q_out, (TT*)k_pool, (TT*)v_pool, cos_t, sin_t, positions, seq_of_token,
-      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout)));
+      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout, interleaved)));
   ALICE_LAUNCH_CHECK();
   return 0;
 }

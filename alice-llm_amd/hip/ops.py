@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA = 0, 1, 2, 3
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 _lock = threading.Lock()
@@ -42,7 +42,8 @@ def _declare(lib) -> None:
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
         "alice_frag16_supported": [I, I, I],
-        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P],
+        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, P],
+        "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
@@ -262,10 +263,12 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
                      v_pool: Optional[torch.Tensor], cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                      positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
                      block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
-                     rotary_dim: int, max_position: int, kv_layout: int = 0) -> None:
+                     rotary_dim: int, max_position: int, kv_layout: int = 0, interleaved: bool = False) -> None:
     """Rotate q and k; write k and v at their positions into the pools [pages, nKV, page, d].
     With k_pool None the row holds q only (num_kv_heads = 0) and nothing is cached.
-    `max_position` is the largest position among `positions` (the host knows it): checked against the tables."""
+    `max_position` is the largest position among `positions` (the host knows it): checked against the tables.
+    interleaved: the q and k heads of qkv hold the rotated pairs (j, j + d/2) at 2j and 2j + 1 (a projection
+    with its rows in that order made them); the outputs are in the plain order either way."""
     T = qkv.shape[0]
     dt = qkv.dtype
     _dev(qkv, "qkv")
@@ -298,7 +301,52 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
     _call("alice_rope_cache_write", qkv.data_ptr(), dtype_code(dt), q_out.data_ptr(), _opt(k_pool, "k_pool"),
           _opt(v_pool, "v_pool"), _opt(cos, "cos"), _opt(sin, "sin"), positions.data_ptr(),
           _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T, row_width, num_heads,
-          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, int(kv_layout), _stream())
+          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, int(kv_layout), int(interleaved), _stream())
+
+
+def linear_rope_cache(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                      block_table: torch.Tensor, *, k_in: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                      max_position: int, kv_layout: int, rows: Optional[int] = None, x_layout: int = LAYOUT_ROW) -> None:
+    """The fused q|k|v projection of at most 64 single tokens with the rotation and the cache write as its
+    epilogue: what linear() followed by rope_cache_write(interleaved=True) gives.  w: the fragment layout of the
+    [(nH + 2 nKV) d, k_in] matrix whose q and k heads have their rows in pair order."""
+    if x_layout == LAYOUT_FRAG16:
+        if rows is None:
+            raise HipLibraryError("activations in fragment order need the number of rows")
+        M = rows
+        _dev(x, "x", torch.bfloat16, (frag_rows(M) * k_in,))
+    else:
+        if x.dim() != 2 or x.shape[1] != k_in:
+            raise HipLibraryError(f"x must be [M, {k_in}], found {tuple(x.shape)}")
+        M = x.shape[0]
+        _dev(x, "x", torch.bfloat16)
+    n_rows = (num_heads + 2 * num_kv_heads) * head_dim
+    _dev(w, "w", torch.bfloat16)
+    need = ((n_rows + 15) // 16 * 16) * ((k_in + 31) // 32 * 32)
+    if w.numel() != need:
+        raise HipLibraryError(f"w in fragment layout must hold {need} elements, found {w.numel()}")
+    _dev(q_out, "q_out", torch.bfloat16, (M, num_heads * head_dim))
+    if k_pool.dim() != 4 or k_pool.shape[1] != num_kv_heads or k_pool.shape[3] != head_dim:
+        raise HipLibraryError(f"k_pool must be [pages, {num_kv_heads}, page, {head_dim}], found {tuple(k_pool.shape)}")
+    _dev(k_pool, "k_pool", torch.bfloat16)
+    _dev(v_pool, "v_pool", torch.bfloat16, k_pool.shape)
+    n_pages, _, page_size, _ = k_pool.shape
+    if cos.dim() != 2 or cos.shape[1] != head_dim // 2 or sin.shape != cos.shape:
+        raise HipLibraryError(f"cos/sin tables must be [positions, {head_dim // 2}]")
+    _dev(cos, "cos", torch.float32)
+    _dev(sin, "sin", torch.float32)
+    if max_position >= cos.shape[0]:
+        raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({cos.shape[0]} positions)")
+    _dev(positions, "positions", torch.int32, (M,))
+    _dev(seq_of_token, "seq_of_token", torch.int32, (M,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"position {max_position} is beyond the block table {tuple(block_table.shape)}")
+    _call("alice_linear_rope_cache", x.data_ptr(), int(x_layout), w.data_ptr(), M, k_in, q_out.data_ptr(), k_pool.data_ptr(),
+          v_pool.data_ptr(), cos.data_ptr(), sin.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(),
+          block_table.data_ptr(), block_table.shape[1], num_heads, num_kv_heads, head_dim, page_size, n_pages,
+          int(kv_layout), _stream())
 
 
 def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor,

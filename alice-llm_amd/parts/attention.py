@@ -66,7 +66,14 @@ class Attention(Part):
         q, k, v = (self._parts.pop(n + "_proj.weight") for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
             q, k, v = q.float(), k.float(), v.float()       # one stored in 32-bit: the fused matrix stays 32-bit
-        self.qkv.load(torch.cat([q, k, v], dim=0))          # rows: all q heads, then k heads, then v heads
+        w = torch.cat([q, k, v], dim=0)                     # rows: all q heads, then k heads, then v heads
+        # a position encoding may ask for the rows of the q and k heads in another order (rotated pairs next to
+        # each other), so that its rotation can be the projection's epilogue
+        order = getattr(self.position, "projection_row_order", lambda *a: None)(self.nH, self.nKV, self.d)
+        self.pair_order = order is not None
+        if self.pair_order:
+            w = w[order.to(w.device)]
+        self.qkv.load(w)
 
     def weight_bytes(self) -> int:
         return self.qkv.nbytes() + self.o.nbytes()
@@ -79,10 +86,15 @@ class Attention(Part):
         """x: [T, H] in the activation dtype (a tensor, or FragmentActs in decode steps); returns the branch
         in float32 ([T, H] or partial sums)."""
         T = x.shape[0]
-        qkv = self.qkv(x, self.precision.act)
         q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
-        self.position.rotate_and_store(qkv, q, ctx, cache, num_heads=self.nH, num_kv_heads=self.nKV,
-                                       head_dim=self.d, kv_layout=self.kv_layout)
+        geometry = dict(num_heads=self.nH, num_kv_heads=self.nKV, head_dim=self.d, kv_layout=self.kv_layout)
+        fused = self.pair_order and self.position.project_rotate_store(self.qkv, x, q, ctx, cache, **geometry)
+        if not fused:
+            qkv = self.qkv(x, self.precision.act)
+            if self.pair_order:
+                self.position.rotate_and_store(qkv, q, ctx, cache, pair_order=True, **geometry)
+            else:
+                self.position.rotate_and_store(qkv, q, ctx, cache, **geometry)
         # Single tokens on the matrix-core kernel: its output goes to the output projection in fragment order.
         frag = (getattr(ctx, "fragment_activations", False) and ctx.is_decode and self.kv_layout == ops.KV_FRAGMENT
                 and self.nH // self.nKV <= 16 and self.o.accepts_fragment_input

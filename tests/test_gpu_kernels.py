@@ -607,6 +607,77 @@ def _rope_fragment_case(nH, nKV, d, lens, starts):
             assert torch.equal(vp[page, h].reshape(-1).cpu()[voff].double(), v[t, h])
 
 
+def pair_order(nH, nKV, d):
+    """Row order of a fused q|k|v projection whose q and k heads have the rotated pairs next to each other."""
+    one = torch.stack([torch.arange(d // 2), torch.arange(d // 2) + d // 2], dim=1).flatten()
+    heads = torch.arange(nH + nKV)[:, None] * d + one[None, :]
+    return torch.cat([heads.flatten(), torch.arange((nH + nKV) * d, (nH + 2 * nKV) * d)])
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nH,nKV,d,T", [(4, 1, 16, 9), (3, 2, 64, 40), (8, 4, 256, 300), (2, 2, 32, 270)])
+@pytest.mark.parametrize("layout", [0, 1])
+def test_rope_takes_pairs_next_to_each_other(dt, nH, nKV, d, T, layout):
+    # the same rows with the pairs (j, j + d/2) at 2j, 2j + 1 give the same bits (both kernels: few and many tokens)
+    if layout == 1 and (dt == "float32" or d % 32):
+        pytest.skip("the fragment cache layout is bfloat16 with head sizes in steps of 32")
+    qkv = rnd(T, (nH + 2 * nKV) * d, seed=50, dtype=DT[dt])
+    pos = torch.arange(T, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    ang = torch.arange(T, dtype=D)[:, None] * 1e4 ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    outs = []
+    for inter in (False, True):
+        kp, vp, bt = paged(T, nKV, d, DT[dt], 1, seed=51)
+        q_out = torch.full((T, nH * d), float("nan"), dtype=DT[dt], device=DEV)
+        src = qkv[:, pair_order(nH, nKV, d).to(DEV)].contiguous() if inter else qkv
+        ops.rope_cache_write(src, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                             rotary_dim=d, max_position=T - 1, kv_layout=layout, interleaved=inter)
+        outs.append((q_out, kp, vp))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("nH,nKV,d,K", [(8, 4, 256, 2304), (3, 1, 64, 96), (4, 2, 128, 320), (2, 2, 16, 72), (16, 16, 128, 64)])
+@pytest.mark.parametrize("M", [1, 7, 16, 33, 64])
+@pytest.mark.parametrize("layout", [0, 1])
+def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K, M, layout):
+    if layout == 1 and d % 32:
+        pytest.skip("the fragment cache layout takes head sizes in steps of 32")
+    N = (nH + 2 * nKV) * d
+    x, w = rnd(M, K, seed=60, dtype=torch.bfloat16), rnd(N, K, seed=61, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w[pair_order(nH, nKV, d).to(DEV)].contiguous())
+    lens = [3 + 37 * b for b in range(M)]                       # every token its own sequence, page and place
+    pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32, device=DEV)
+    seq = torch.randperm(M, generator=torch.Generator().manual_seed(1)).to(torch.int32).to(DEV)
+    ang = torch.arange(max(lens), dtype=D)[:, None] * 1e4 ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    res = []
+    for fused in (False, True):
+        for frag_in in ((False, True) if fused and K % 32 == 0 else (False,)):
+            kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, M, seed=62)
+            q_out = torch.full((M, nH * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+            if fused:
+                xin = acts_to_fragments(x) if frag_in else x
+                ops.linear_rope_cache(xin, wf, q_out, kp, vp, cos, sin, pos, seq, bt, k_in=K, num_heads=nH, num_kv_heads=nKV,
+                                      head_dim=d, max_position=max(lens) - 1, kv_layout=layout, rows=M,
+                                      x_layout=ops.LAYOUT_FRAG16 if frag_in else ops.LAYOUT_ROW)
+            else:
+                qkv = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+                ops.linear(x, wf, qkv, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False)
+                ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                                     rotary_dim=d, max_position=max(lens) - 1, kv_layout=layout, interleaved=True)
+            res.append((q_out, kp, vp))
+    for other in res[1:]:
+        for a, b in zip(res[0], other):
+            assert torch.equal(a, b)
+    # and the separate kernels against the plain formulas, from the rows in their plain order
+    qkv_ref = x.double().cpu() @ w.double().cpu().T
+    qkv_ref = qkv_ref.to(torch.bfloat16).double()
+    q_ref = P.rope_half_split(qkv_ref[:, :nH * d].view(M, nH, d), pos.cpu(), 1e4)
+    close(res[0][0].view(M, nH, d), q_ref, 2 ** -5, 2 ** -6)
+
+
 @pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
 @pytest.mark.parametrize("cap,window", [(None, None), (5.0, 50), (50.0, 7), (2.0, 64)])
 def test_attention_mfma_prompts(nH, nKV, d, cap, window):

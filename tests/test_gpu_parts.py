@@ -255,6 +255,9 @@ def toy_plain(model, tokens):
             a = torch.stack(outs) @ m.w["out.weight"].double().cpu().T
         else:
             W = m.qkv.weight.double().cpu()
+            order = m.position.projection_row_order(2, 1, 16)     # the fused rows may be in the rotation's pair order
+            if m.pair_order:
+                W = torch.empty_like(W).index_copy_(0, order, W)
             q = (h @ W[:32].T).view(T, 2, 16)
             if e.cache_from is None:
                 k = P.rope_half_split((h @ W[32:48].T).view(T, 1, 16), torch.arange(T), 100.0)
