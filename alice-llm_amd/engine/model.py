@@ -132,5 +132,8 @@ class CausalLM:
             stream.flush()
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
         frag = getattr(ctx, "fragment_activations", False) and getattr(self.head, "accepts_fragment_activations", False)
-        normed = stream.rows_normed(self.final_norm, ctx.want_rows, fragments=frag)
+        if getattr(ctx, "want_every_row", False):
+            normed = stream.normed(self.final_norm, fragments=frag)        # the last add and the norm as one kernel
+        else:
+            normed = stream.rows_normed(self.final_norm, ctx.want_rows, fragments=frag)
         return self.head.forward(normed)
