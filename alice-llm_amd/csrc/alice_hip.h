@@ -64,8 +64,8 @@ int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool
                            int row_width, int nH, int nKV, int d, int rotary_dim, int page_size, int n_pages,
                            int kv_layout, int interleaved, hipStream_t stream);
 
-// The fused q|k|v projection of single tokens (at most 64), with the rotation and the cache write as its
-// epilogue: x [M, K] (row-major or fragment order), W in the fragment layout with the rows of every q and k
+// The fused q|k|v projection with the rotation and the cache write as its epilogue (single tokens: the
+// streaming kernel; more than 64 tokens: the tiled one): x [M, K] (row-major or fragment order), W in the fragment layout with the rows of every q and k
 // head in pair order (rows j and j + d/2 of a head at 2j and 2j + 1).  Writes what alice_linear followed by
 // alice_rope_cache_write (interleaved) would: q_out [M, nH * d] and the token's keys and values in the cache.
 int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, int K, void* q_out, void* k_pool,

@@ -15,3 +15,10 @@ __device__ __forceinline__ size_t v_offset(int layout, int t, int e, int d) {
   const int tt = t & 31, w = tt & 15;
   return ((size_t)((t >> 5) * (d >> 4) + (e >> 4)) * 64 + (w >> 2) * 16 + (e & 15)) * 8 + ((tt >> 4) * 4 + (w & 3));
 }
+
+// The rotation of one pair, written with explicit roundings so that every kernel that rotates (the separate
+// kernels for few and for many tokens, the projections' epilogue) gives the same bits.
+__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float& y0, float& y1) {
+  y0 = fmaf(x0, c, -__fmul_rn(x1, s));
+  y1 = fmaf(x0, s, __fmul_rn(x1, c));
+}

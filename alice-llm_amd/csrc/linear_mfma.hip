@@ -99,6 +99,56 @@ struct RopeArgs {
   int bt_stride, nH, nKV, d, page_size, n_pages, layout;
 };
 
+// Where token m's keys and values go.
+struct RopeToken {
+  int pos, tp;
+  bool page_ok;
+  size_t page_base;
+};
+__device__ __forceinline__ RopeToken rope_token(const RopeArgs& ra, int m) {
+  RopeToken t;
+  t.pos = ra.positions[m];
+  t.tp = t.pos % ra.page_size;
+  const int page = ra.block_table[(size_t)ra.seq_of_token[m] * ra.bt_stride + t.pos / ra.page_size];
+  t.page_ok = page >= 0 && page < ra.n_pages;
+  t.page_base = (size_t)(t.page_ok ? page : 0) * ra.nKV * ra.page_size * ra.d;
+  return t;
+}
+// The rotation epilogue for four consecutive output features n .. n+3 (in W's row order) of token m.  The
+// rows of W are all q heads, all k heads, all v heads, the rows of every q and k head in pair order: the four
+// features are two whole rotated pairs (or four elements of a value head).  The sums are rounded to bfloat16
+// before the rotation, as they are when the projection and the rotation are separate kernels: both ways give
+// the same bits.
+__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc) {
+  const int d = ra.d, half = d >> 1;
+  const int head = n / d, w = n % d;
+  float x[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[e]);
+  if (head < ra.nH + ra.nKV) {
+    const int p0 = w >> 1;                                 // the pairs p0 and p0 + 1 of the head
+    const float2 c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)t.pos * half + p0);
+    const float2 sn = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)t.pos * half + p0);
+    float l0, h0, l1, h1;
+    rotate_pair(x[0], x[1], c.x, sn.x, l0, h0);
+    rotate_pair(x[2], x[3], c.y, sn.y, l1, h1);
+    const uint32_t lo = pack_bf16x2(l0, l1), hi = pack_bf16x2(h0, h1);
+    if (head < ra.nH) {
+      bf16_t* dst = ra.q_out + ((size_t)m * ra.nH + head) * d;
+      *reinterpret_cast<uint32_t*>(dst + p0) = lo;
+      *reinterpret_cast<uint32_t*>(dst + p0 + half) = hi;
+    } else if (t.page_ok) {
+      bf16_t* dst = ra.k_pool + t.page_base + (size_t)(head - ra.nH) * ra.page_size * d;
+      *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, t.tp, p0, d)) = lo;
+      *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, t.tp, p0 + half, d)) = hi;
+    }
+  } else if (t.page_ok) {
+    bf16_t* dst = ra.v_pool + t.page_base + (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[v_offset(ra.layout, t.tp, w + e, d)] = f32_to_bf16(x[e]);
+  }
+}
+
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
 // Block: NW waves on the same RT row tiles; wave w takes k-tiles kb + w, kb + w + NW, ...; the parts of
 // waves 1.. go through LDS and wave 0 adds them in the order 1, 2, 3, ....  grid.x: groups of RT row
@@ -223,49 +273,13 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
       }
 
   if constexpr (EPI == ALICE_EPI_ROPE) {
-    // The rows of W are all q heads, all k heads, all v heads, the rows of every q and k head in pair order:
-    // this lane's four features of a tile are two whole rotated pairs (or four elements of a value head).
-    // The sums are rounded to bfloat16 before the rotation, as they are when the projection and the
-    // rotation are separate kernels: both ways give the same bits.
-    const int d = ra.d, half = d >> 1;
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       if (!row_ok[j]) continue;
-      const int m = row[j];
-      const int pos = ra.positions[m];
-      const int tp = pos % ra.page_size;
-      const int page = ra.block_table[(size_t)ra.seq_of_token[m] * ra.bt_stride + pos / ra.page_size];
-      const bool page_ok = page >= 0 && page < ra.n_pages;
-      const size_t page_base = (size_t)(page_ok ? page : 0) * ra.nKV * ra.page_size * d;
+      const RopeToken t = rope_token(ra, row[j]);
 #pragma unroll
-      for (int i = 0; i < RT; ++i) {
-        if (tile[i] >= NT) continue;
-        const int n = tile[i] * 16 + g * 4;                // first of this lane's four features, in W's row order
-        const int head = n / d, w = n % d;
-        float x[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[i][j][e]);
-        if (head < ra.nH + ra.nKV) {
-          const int p0 = w >> 1;                           // the pairs p0 and p0 + 1 of the head
-          const float2 c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)pos * half + p0);
-          const float2 sn = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)pos * half + p0);
-          const uint32_t lo = pack_bf16x2(x[0] * c.x - x[1] * sn.x, x[2] * c.y - x[3] * sn.y);
-          const uint32_t hi = pack_bf16x2(x[0] * sn.x + x[1] * c.x, x[2] * sn.y + x[3] * c.y);
-          if (head < ra.nH) {
-            bf16_t* dst = ra.q_out + ((size_t)m * ra.nH + head) * d;
-            *reinterpret_cast<uint32_t*>(dst + p0) = lo;
-            *reinterpret_cast<uint32_t*>(dst + p0 + half) = hi;
-          } else if (page_ok) {
-            bf16_t* dst = ra.k_pool + page_base + (size_t)(head - ra.nH) * ra.page_size * d;
-            *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, tp, p0, d)) = lo;
-            *reinterpret_cast<uint32_t*>(dst + k_offset(ra.layout, tp, p0 + half, d)) = hi;
-          }
-        } else if (page_ok) {
-          bf16_t* dst = ra.v_pool + page_base + (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) dst[v_offset(ra.layout, tp, w + e, d)] = f32_to_bf16(x[e]);
-        }
-      }
+      for (int i = 0; i < RT; ++i)
+        if (tile[i] < NT) rope_store4(ra, row[j], t, tile[i] * 16 + g * 4, acc[i][j]);
     }
     return;
   }
@@ -319,7 +333,7 @@ constexpr int KC = 2;      // k-tiles per stage
 template <int EPI, typename TO, bool FULL, int TM, bool XF>
 __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                               float epi, int gx, int gy, int kt_per_slice) {
+                                                               float epi, int gx, int gy, int kt_per_slice, RopeArgs ra) {
   constexpr int XJ = TM / 4;                               // token tiles each wave stages
   __shared__ __align__(16) uint32_t xs_raw[2 * KC * TM * 64 * 4];
   u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
@@ -434,6 +448,18 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
     stage_mfma(S - 1, false);
   }
 
+  if constexpr (EPI == ALICE_EPI_ROPE) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + j * 16 + r;
+      if (m >= M) continue;
+      const RopeToken t = rope_token(ra, m);
+#pragma unroll
+      for (int i = 0; i < WN; ++i)
+        if (tile[i] < NT) rope_store4(ra, m, t, tile[i] * 16 + g * 4, acc[i][j]);
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
     const int m = m0 + j * 16 + r;
@@ -534,7 +560,7 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
 
 template <int EPI, typename TO>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
-                 hipStream_t s) {
+                 hipStream_t s, const RopeArgs& ra = RopeArgs{}) {
   (void)y_frag;
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
@@ -545,14 +571,14 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
     if (x_frag) {
       // fragment order is what decode steps use: few tokens, one or a few block rows
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 8, true><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+      linear_tiled_lds_kernel<EPI, TO, false, 8, true><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
     } else if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 8, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+      linear_tiled_lds_kernel<EPI, TO, false, 8, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
     } else {
       gy = ceil_div(M, 64);
       dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 4, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per);
+      linear_tiled_lds_kernel<EPI, TO, false, 4, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
     }
   }
   ALICE_LAUNCH_CHECK();
@@ -651,7 +677,7 @@ extern "C" int alice_linear_rope_cache(const void* x, int x_layout, const void* 
                                        void* v_pool, const float* cos_t, const float* sin_t, const int* positions,
                                        const int* seq_of_token, const int* block_table, int bt_stride, int nH, int nKV,
                                        int d, int page_size, int n_pages, int kv_layout, hipStream_t stream) {
-  ALICE_CHECK(M >= 0 && M <= 64, "linear+rope: at most 64 tokens, found %d", M);
+  ALICE_CHECK(M >= 0 && ceil_div(M, 128) <= 65535, "linear+rope: bad number of tokens %d", M);
   ALICE_CHECK(K > 0 && K % 8 == 0, "linear+rope: K must be a multiple of 8, found %d", K);
   ALICE_CHECK(nH >= 1 && nKV >= 1 && d >= 16 && d % 16 == 0, "linear+rope: bad heads nH=%d nKV=%d d=%d (d must be a multiple of 16)", nH, nKV, d);
   ALICE_CHECK(x && w && q_out && k_pool && v_pool && cos_t && sin_t && positions && seq_of_token && block_table,
@@ -668,6 +694,7 @@ extern "C" int alice_linear_rope_cache(const void* x, int x_layout, const void* 
   RopeArgs ra{(bf16_t*)q_out, (bf16_t*)k_pool, (bf16_t*)v_pool, cos_t, sin_t, positions, seq_of_token, block_table,
               bt_stride, nH, nKV, d, page_size, n_pages, kv_layout};
   const int x_frag = x_layout == ALICE_LAYOUT_FRAG16;
+  if (M > 64) return launch_tiled<ALICE_EPI_ROPE, bf16_t>(x, w, nullptr, M, N, K, 1, 0.f, x_frag, 0, stream, ra);
   const int rt = skinny_row_tiles(M, N, ALICE_EPI_NONE, 1, K);
 #define GO(RT, MT) return launch_skinny<RT, MT, ALICE_EPI_ROPE, bf16_t>(x, w, nullptr, M, N, K, 1, 0.f, x_frag, 0, stream, ra)
 #define BY_RT(MT)                \

@@ -54,9 +54,10 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
       // the rotated pair (j, j + half) if j < half; elements at or beyond R pass through, spread over the items
       if (j < half) {
         float x0 = load_f32(src, interleaved ? 2 * j : j), x1 = load_f32(src, interleaved ? 2 * j + 1 : j + half);
-        float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f;
-        store_f32(dst, at(j), x0 * c - x1 * s);
-        store_f32(dst, at(j + half), x0 * s + x1 * c);
+        float c = cs ? cs[j] : 1.f, s = sn ? sn[j] : 0.f, y0, y1;
+        rotate_pair(x0, x1, c, s, y0, y1);
+        store_f32(dst, at(j), y0);
+        store_f32(dst, at(j + half), y1);
       }
       for (int e = R + j; e < d; e += hd2) store_f32(dst, at(e), load_f32(src, e));
     }
@@ -124,9 +125,11 @@ __global__ void rope_cache_vec_kernel(const bf16_t* __restrict__ qkv, bf16_t* __
       for (int p = 0; p < 4; ++p) {
         const float a0 = bf16_bits_to_f32(lw[p] & 0xffffu), a1 = bf16_bits_to_f32(lw[p] >> 16);
         const float b0 = bf16_bits_to_f32(hw[p] & 0xffffu), b1 = bf16_bits_to_f32(hw[p] >> 16);
-        // the same expressions as the scalar kernel's, so both round alike
-        ol[p] = (uint32_t)f32_to_bf16(a0 * c[2 * p] - b0 * sv[2 * p]).bits | ((uint32_t)f32_to_bf16(a1 * c[2 * p + 1] - b1 * sv[2 * p + 1]).bits << 16);
-        oh[p] = (uint32_t)f32_to_bf16(a0 * sv[2 * p] + b0 * c[2 * p]).bits | ((uint32_t)f32_to_bf16(a1 * sv[2 * p + 1] + b1 * c[2 * p + 1]).bits << 16);
+        float l0, h0, l1, h1;
+        rotate_pair(a0, b0, c[2 * p], sv[2 * p], l0, h0);
+        rotate_pair(a1, b1, c[2 * p + 1], sv[2 * p + 1], l1, h1);
+        ol[p] = pack_bf16x2(l0, l1);
+        oh[p] = pack_bf16x2(h0, h1);
       }
       bf16_t* dst;
       size_t o_lo, o_hi;

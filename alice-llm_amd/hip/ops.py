@@ -308,8 +308,7 @@ def linear_rope_cache(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, k_p
                       cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
                       block_table: torch.Tensor, *, k_in: int, num_heads: int, num_kv_heads: int, head_dim: int,
                       max_position: int, kv_layout: int, rows: Optional[int] = None, x_layout: int = LAYOUT_ROW) -> None:
-    """The fused q|k|v projection of at most 64 single tokens with the rotation and the cache write as its
-    epilogue: what linear() followed by rope_cache_write(interleaved=True) gives.  w: the fragment layout of the
+    """The fused q|k|v projection with the rotation and the cache write as its epilogue: what linear() followed by rope_cache_write(interleaved=True) gives.  w: the fragment layout of the
     [(nH + 2 nKV) d, k_in] matrix whose q and k heads have their rows in pair order."""
     if x_layout == LAYOUT_FRAG16:
         if rows is None:

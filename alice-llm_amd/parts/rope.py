@@ -60,11 +60,11 @@ class RotaryEncoding(Part):
 
     def project_rotate_store(self, proj, x, q_out: torch.Tensor, ctx, cache, *, num_heads: int, num_kv_heads: int,
                              head_dim: int, kv_layout: int) -> bool:
-        """Single tokens: projection (a Linear in the fragment layout with its rows in pair order), rotation and
-        cache write as one kernel.  False where that kernel does not apply; the caller then takes the steps apart."""
+        """Projection (a Linear in the fragment layout with its rows in pair order), rotation and cache write as
+        one kernel.  False where that kernel does not apply; the caller then takes the steps apart."""
         from .base import FragmentActs
         frag_in = isinstance(x, FragmentActs)
-        if not (ctx.is_decode and ctx.n_tokens <= 64 and cache is not None and cache.writable
+        if not (cache is not None and cache.writable
                 and proj.layout == ops.LAYOUT_FRAG16 and proj.precision.act == torch.bfloat16 and head_dim % 16 == 0
                 and (kv_layout == ops.KV_ROW or head_dim % 32 == 0)):
             return False

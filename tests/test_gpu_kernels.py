@@ -639,7 +639,7 @@ def test_rope_takes_pairs_next_to_each_other(dt, nH, nKV, d, T, layout):
 
 
 @pytest.mark.parametrize("nH,nKV,d,K", [(8, 4, 256, 2304), (3, 1, 64, 96), (4, 2, 128, 320), (2, 2, 16, 72), (16, 16, 128, 64)])
-@pytest.mark.parametrize("M", [1, 7, 16, 33, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 33, 64, 130, 300])
 @pytest.mark.parametrize("layout", [0, 1])
 def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K, M, layout):
     if layout == 1 and d % 32:
@@ -647,15 +647,18 @@ def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K,
     N = (nH + 2 * nKV) * d
     x, w = rnd(M, K, seed=60, dtype=torch.bfloat16), rnd(N, K, seed=61, scale=0.1, dtype=torch.bfloat16)
     wf = ops.to_frag16(w[pair_order(nH, nKV, d).to(DEV)].contiguous())
-    lens = [3 + 37 * b for b in range(M)]                       # every token its own sequence, page and place
-    pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32, device=DEV)
-    seq = torch.randperm(M, generator=torch.Generator().manual_seed(1)).to(torch.int32).to(DEV)
+    # up to five sequences that start at different places; consecutive tokens go to different sequences
+    n_seq, starts = min(M, 5), [0, 60, 100, 7, 33]
+    order = torch.randperm(n_seq, generator=torch.Generator().manual_seed(1)).tolist()
+    pos = torch.tensor([starts[t % n_seq] + t // n_seq for t in range(M)], dtype=torch.int32, device=DEV)
+    seq = torch.tensor([order[t % n_seq] for t in range(M)], dtype=torch.int32, device=DEV)
+    lens = [int(pos.max()) + 1]
     ang = torch.arange(max(lens), dtype=D)[:, None] * 1e4 ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
     cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
     res = []
     for fused in (False, True):
         for frag_in in ((False, True) if fused and K % 32 == 0 else (False,)):
-            kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, M, seed=62)
+            kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, n_seq, seed=62)
             q_out = torch.full((M, nH * d), float("nan"), dtype=torch.bfloat16, device=DEV)
             if fused:
                 xin = acts_to_fragments(x) if frag_in else x
