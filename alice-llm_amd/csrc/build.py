@@ -81,7 +81,9 @@ def build(verbose: bool = True) -> str:
     srcs = sources()
     if verbose:
         _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
-    objs = {s: os.path.join(obj_dir, s[:-4] + ".o") for s in srcs}
+    # object files carry the process id: two processes that build at once (a test runner and a program it
+    # starts) do not write into each other's files; the library itself is put in place by a rename
+    objs = {s: os.path.join(obj_dir, f"{s[:-4]}.{os.getpid()}.o") for s in srcs}
     t0 = time.time()
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or (os.cpu_count() or 4), 16))
     with cf.ThreadPoolExecutor(workers) as pool:
@@ -99,6 +101,11 @@ def build(verbose: bool = True) -> str:
     tmp = lib + f".tmp{os.getpid()}"
     r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp, *objs.values()],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    for o in objs.values():
+        try:
+            os.remove(o)
+        except OSError:
+            pass
     if r.returncode != 0:
         raise RuntimeError(f"linking {LIB_NAME} failed:\n{r.stderr[-4000:]}")
     os.replace(tmp, lib)
