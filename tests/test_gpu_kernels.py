@@ -320,15 +320,67 @@ def test_sample_matches_plain(V):
     g = torch.Generator().manual_seed(14)
     for temperature, top_k, top_p in ((0.8, 0, 1.0), (1.5, 40, 1.0), (0.7, 0, 0.9), (1.0, 50, 0.5), (1e-3, 0, 1.0)):
         u = torch.rand(B, generator=g)
-        got = ops.sample(logits, u.to(DEV), temperature, top_k, top_p).cpu().tolist()
-        for b in range(B):
-            want = P.plain_sample(logits[b].double().cpu(), temperature, top_k, top_p, float(u[b]))
-            if got[b] != want:
-                # a draw within rounding of a boundary of the cumulative sum may fall on either side
-                x = logits[b].double().cpu() / temperature
-                x = P.plain_top_p(P.plain_top_k(x, top_k), top_p)
-                cdf = torch.cumsum(P.plain_softmax(x), 0)
-                assert x[got[b]] > -math.inf and abs(float(cdf[min(got[b], want)]) - float(u[b])) < 1e-5, (b, got[b], want)
+        check_samples(logits, u, temperature, top_k, top_p)
+
+
+def top_p_ties_kept(x, p):
+    """plain_top_p, and every value tied with the last kept one as well: what the kernel's threshold keeps."""
+    kept = P.plain_top_p(x, p)
+    return torch.where(x >= kept[kept > -math.inf].min(), x, torch.full_like(x, -math.inf))
+
+
+def check_samples(logits, u, temperature, top_k, top_p):
+    got = ops.sample(logits, u.to(DEV), temperature, top_k, top_p).cpu().tolist()
+    for b in range(logits.shape[0]):
+        x = top_p_ties_kept(P.plain_top_k(logits[b].double().cpu() / temperature, top_k), top_p)
+        probs = P.plain_softmax(x)
+        want = P.plain_inverse_cdf(probs, float(u[b]))
+        if got[b] != want:
+            # a draw within rounding of a boundary of the cumulative sum may fall on either side
+            cdf = torch.cumsum(probs, 0)
+            assert x[got[b]] > -math.inf and abs(float(cdf[min(got[b], want)]) - float(u[b])) < 1e-5, (b, got[b], want)
+    return got
+
+
+@pytest.mark.parametrize("V", [383, 5000, 70002])
+def test_sample_where_the_kept_set_is_large_or_tied(V):
+    """Rows whose kept set does not fit the kernel's short list, and ties at both thresholds."""
+    g = torch.Generator().manual_seed(16)
+    B = 5
+    flat = torch.zeros(B, V)                                          # every token tied
+    steps = torch.randint(0, 3, (B, V), generator=g).float()          # three values, thousands of ties each
+    peaks = rnd(B, V, seed=17, scale=0.1).cpu()
+    peaks[:, 11] = peaks[:, V - 2] = 9.0                              # two tied peaks far above a flat rest
+    holes = rnd(B, V, seed=18, scale=3.0).cpu()
+    holes[:, ::3] = -math.inf                                         # masked tokens are never drawn
+    wide = rnd(B, V, seed=19, scale=0.5).cpu()                        # a nucleus of most of the vocabulary
+    for logits in (flat, steps, peaks, holes, wide):
+        logits = logits.to(DEV)
+        for temperature, top_k, top_p in ((1.0, 0, 0.9), (1.0, 7, 1.0), (0.9, V - 1, 0.95), (1.3, 6000, 0.999),
+                                          (1.0, 2, 0.6), (0.5, 0, 0.3)):
+            u = torch.rand(B, generator=g)
+            got = check_samples(logits, u, temperature, top_k, top_p)
+            assert all(logits[b, t] > -math.inf for b, t in enumerate(got))
+    u = torch.tensor([0.1, 0.3, 0.5, 0.7, 0.9])
+    assert set(ops.sample(peaks.to(DEV), u.to(DEV), 1.0, 2, 1.0).cpu().tolist()) == {11, V - 2}
+    assert set(ops.sample(peaks.to(DEV), u.to(DEV), 1.0, 1, 1.0).cpu().tolist()) == {11, V - 2}   # ties are kept
+
+
+def test_sample_depends_on_the_row_alone():
+    """The same row gives the same token wherever it stands in the batch, whatever the other rows hold."""
+    V = 70002
+    row = rnd(1, V, seed=20, scale=2.0)
+    other = rnd(7, V, seed=21, scale=5.0)
+    g = torch.Generator().manual_seed(22)
+    for temperature, top_k, top_p in ((1.0, 0, 1.0), (0.8, 40, 0.9), (1.2, 0, 0.95), (1.0, 30000, 0.9)):
+        for _ in range(4):
+            u = float(torch.rand(1, generator=g))
+            alone = ops.sample(row, torch.tensor([u], device=DEV), temperature, top_k, top_p).item()
+            for place in (0, 3, 7):
+                batch = torch.cat([other[:place], row, other[place:]])
+                us = torch.rand(8, generator=g)
+                us[place] = u
+                assert ops.sample(batch, us.to(DEV), temperature, top_k, top_p)[place].item() == alone
 
 
 def test_sample_frequencies():
