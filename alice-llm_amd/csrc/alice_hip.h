@@ -17,6 +17,8 @@
 #define ALICE_PREFILL_AUTO 0    // prompt attention: chosen by the grid's size
 #define ALICE_PREFILL_TILES 1   // a wave takes whole tiles of 16 queries (two heads where the group is even)
 #define ALICE_PREFILL_SPLIT 2   // the four waves of a block split one tile's keys
+#define ALICE_PREFILL_SHARED4 3 // the four waves of a block share each block of keys and values through LDS
+#define ALICE_PREFILL_SHARED8 4 // the same with eight waves
 
 #define ALICE_LINEAR_AUTO 0
 #define ALICE_LINEAR_GENERIC 1

@@ -101,7 +101,6 @@ struct Core {
   template <bool SOFTCAP>
   __device__ __forceinline__ void scores(const u32x4 (&kf)[2][DT], int key0, const int* pos, int window, ScoreConsts k,
                                          int lane, u32x4 (&p)[NB]) {
-    const int g = lane >> 4;
     f32x4 s[NB][2];
 #pragma unroll
     for (int b = 0; b < NB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -111,6 +110,52 @@ struct Core {
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int b = 0; b < NB; ++b) s[b][t] = mfma16(kf[t][dt], q[b][dt], s[b][t]);
+    softmax_step<SOFTCAP>(s, key0, pos, window, k, lane, p);
+  }
+
+  // The same with the key and value fragments of the block in LDS (laid out as in the cache: keys
+  // [2][DT][64 lanes][8], values [2 DT][64 lanes][8]).
+  template <bool SOFTCAP>
+  __device__ __forceinline__ void compute_lds(const u32x4* __restrict__ kl, const u32x4* __restrict__ vl, int key0,
+                                              const int* pos, int window, ScoreConsts k, int lane) {
+    // All reads of a phase are issued before its products (the scheduling barriers keep them there: left alone,
+    // the compiler reads one fragment at a time into the same registers and waits for each).  The first half of
+    // the values is read before the softmax arithmetic and arrives during it.
+    u32x4 f[2 * DT];
+#pragma unroll
+    for (int i = 0; i < 2 * DT; ++i) f[i] = kl[i * 64 + lane];              // keys: tile i / DT, d tile i % DT
+    __builtin_amdgcn_sched_barrier(0);
+    f32x4 s[NB][2];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) s[b][0] = s[b][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        s[b][0] = mfma16(f[dt], q[b][dt], s[b][0]);
+        s[b][1] = mfma16(f[DT + dt], q[b][dt], s[b][1]);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) f[t] = vl[t * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 p[NB];
+    softmax_step<SOFTCAP>(s, key0, pos, window, k, lane, p);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = DT; t < 2 * DT; ++t) f[t] = vl[t * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) o[b][t] = mfma16(f[t], p[b], o[b][t]);
+  }
+
+  // From the raw dot products of 32 keys to their probabilities (see scores()).
+  template <bool SOFTCAP>
+  __device__ __forceinline__ void softmax_step(f32x4 (&s)[NB][2], int key0, const int* pos, int window, ScoreConsts k,
+                                               int lane, u32x4 (&p)[NB]) {
+    const int g = lane >> 4;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       // key visible iff lo <= key <= pos, i.e. (unsigned)(key - lo) <= (unsigned)(pos - lo); no query: span 0 and rel > 0
@@ -359,6 +404,104 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
   }
 }
 
+// Prompts, third form: the NW (4 or 8) waves of a block share every block of 32 keys and values through LDS.
+// A block takes the heads of one kv head (1, 2 or 4 of them at a time: HB) for 16 NW / HB tokens; wave w takes
+// head w % HB and tokens 16 (w / HB) .. +15 of the block's.  A block of keys and values is a contiguous copy
+// of the cache's fragment order, so filling LDS and reading fragments from it are both linear.  Two buffers:
+// the next block is on its way from memory into registers while this one is computed, and one barrier a
+// step suffices.  Against whole tiles per wave, memory traffic falls by the number of waves.
+// grid: (tiles of 16 NW / HB tokens, from the end backwards; sequences; kv heads x passes over the group).
+template <int DT, bool SOFTCAP, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int HB) {
+  constexpr int D = DT * 32;
+  constexpr int NT = 64 * NW;
+  constexpr int PIECES = 4 * DT * 64;                        // 16-byte pieces of a block: keys, then values
+  constexpr int CH = (PIECES + NT - 1) / NT;                 // pieces per thread
+  extern __shared__ __align__(16) uint32_t kv_raw[];         // [2 buffers][keys 2 DT KB | values 2 DT KB]
+  u32x4* kv = reinterpret_cast<u32x4*>(kv_raw);
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col = lane & 15, g = lane >> 4;
+  const int group = nH / nKV, passes = (group + HB - 1) / HB;
+  const int b = blockIdx.y, kvh = blockIdx.z / passes, hh = (blockIdx.z % passes) * HB + wave % HB;
+  const int tokens = 16 * NW / HB;
+  const int t_begin = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_begin;
+  const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int block_first = tile * tokens;                     // first token of the block among the sequence's new ones
+  if (block_first >= n_new) return;                          // the whole block
+  const int start_len = context_lens[b] - n_new;
+  const int first = block_first + (wave / HB) * 16;
+  const bool wave_ok = first < n_new && hh < group;
+  const int my_tok = first + col;
+  const bool tok_ok = wave_ok && my_tok < n_new;
+  int pos[1] = {tok_ok ? start_len + my_tok : -1};
+  const int* bt = block_table + (size_t)b * bt_stride;
+  const size_t page_elems = (size_t)64 * D;
+  const ScoreConsts sc(scale, cap);
+  // the block's run of key blocks, and this wave's own within it
+  const int block_last_pos = start_len + min(block_first + tokens, n_new) - 1;
+  const int kb_begin = (window > 0 ? max(0, start_len + block_first + 1 - window) : 0) >> 5, kb_end = block_last_pos >> 5;
+  const int my_begin = (window > 0 ? max(0, start_len + first + 1 - window) : 0) >> 5;
+  const int my_end = wave_ok ? (start_len + min(first + 15, n_new - 1)) >> 5 : -1;
+
+  Core<DT, 1> c;
+  c.init();
+  {
+    const bf16_t* qrow = q + ((size_t)(t_begin + (tok_ok ? my_tok : 0)) * nH + kvh * group + (hh < group ? hh : 0)) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      c.q[0][dt] = u32x4{0u, 0u, 0u, 0u};
+      if (tok_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
+    }
+  }
+  // piece j of a thread: piece threadIdx.x + NT j of the block.  Loads are unconditional: past the last block
+  // the last one is fetched again, and a piece past the end is the last piece.
+  u32x4 st[CH];
+  auto fetch = [&](int kb32) {
+    kb32 = min(kb32, kb_end);
+    const int page = bt[kb32 >> 1];
+    const u32x4* kp = reinterpret_cast<const u32x4*>(k_pool + ((size_t)page * nKV + kvh) * page_elems) + (size_t)(kb32 & 1) * 2 * DT * 64;
+    const u32x4* vp = reinterpret_cast<const u32x4*>(v_pool + ((size_t)page * nKV + kvh) * page_elems) + (size_t)(kb32 & 1) * 2 * DT * 64;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int piece = min((int)threadIdx.x + NT * j, PIECES - 1);
+      st[j] = *(piece < 2 * DT * 64 ? kp + piece : vp + (piece - 2 * DT * 64));
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int piece = (int)threadIdx.x + NT * j;
+      if (PIECES % NT == 0 || piece < PIECES) kv[(size_t)buf * PIECES + piece] = st[j];
+    }
+  };
+  fetch(kb_begin);
+  put(0);
+  __syncthreads();
+  for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
+    const int buf = (kb32 - kb_begin) & 1;
+    fetch(kb32 + 1);
+    if (kb32 >= my_begin && kb32 <= my_end) {
+      const u32x4* kl = kv + (size_t)buf * PIECES;
+      c.template compute_lds<SOFTCAP>(kl, kl + 2 * DT * 64, kb32 << 5, pos, window, sc, lane);
+    }
+    put(buf ^ 1);
+    __syncthreads();
+  }
+  c.finish();
+  if (!tok_ok) return;
+  const float inv = 1.f / c.l[0];
+  bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + kvh * group + hh) * D;
+#pragma unroll
+  for (int t = 0; t < 2 * DT; ++t) {
+    const f32x4 v = c.o[0][t] * inv;
+    uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+    *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+  }
+}
+
 // Where output element (sequence b, column c of nH * D) goes: row-major, or fragment order for the output
 // projection's streaming kernel ([B/16][nH*D/32][64][8]).
 __device__ __forceinline__ size_t decode_out_index(int layout, int b, int c, int width) {
@@ -519,7 +662,7 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   // Two heads a wave halve the key/value reads.
   const long waves2 = (long)ceil_div(max_new, 64) * B * nKV * ceil_div(group, 2) * 4;
   const int gh = group % 2 == 0 ? 2 : 1;
-  ALICE_CHECK(variant >= 0 && variant <= 2, "attention: unknown variant %d", variant);
+  ALICE_CHECK(variant >= 0 && variant <= 4, "attention: unknown variant %d", variant);
   ALICE_CHECK((long)nKV * ceil_div(group, gh) <= 65535, "attention: too many heads for one launch");
   dim3 grid(ceil_div(max_new, 64), B, nKV * ceil_div(group, gh));
 #define GO(DT, GH)                                                                                                          \
@@ -544,6 +687,34 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   } while (0)
   // Few waves (one prompt of a few thousand tokens): split every tile's keys over four waves.  Many: whole
   // tiles per wave, two heads a wave where the group is even.
+#define GOL(DT, NW)                                                                                                         \
+  do {                                                                                                                      \
+    const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);                                                           \
+    ALICE_CHECK((long)nKV * ceil_div(group, hb) <= 65535, "attention: too many heads for one launch");                      \
+    dim3 lgrid(ceil_div(max_new, 16 * NW / hb), B, nKV * ceil_div(group, hb));                                              \
+    const size_t lds = (size_t)2 * 4 * DT * 1024;                                                                           \
+    if (softcap > 0.f)                                                                                                      \
+      attn_prefill_shared_kernel<DT, true, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb);             \
+    else                                                                                                                    \
+      attn_prefill_shared_kernel<DT, false, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb);             \
+  } while (0)
+  // Which form (measured on Gemma 2 shapes): with many blocks, four waves sharing their keys; with fewer, eight
+  // (half as many blocks, half the key traffic); with too few blocks to fill the chip, one tile's keys split
+  // over a block's waves.  Small heads spend their time in the softmax arithmetic and gain nothing from sharing.
+  if (variant == ALICE_PREFILL_AUTO && d >= 128) {
+    const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+    const long per_tile = (long)B * nKV * ceil_div(group, hb);
+    if (per_tile * ceil_div(max_new, 64 / hb) >= 2048) variant = ALICE_PREFILL_SHARED4;
+    else if (per_tile * ceil_div(max_new, 128 / hb) >= 192) variant = ALICE_PREFILL_SHARED8;
+  }
+  if (variant == ALICE_PREFILL_SHARED4 || variant == ALICE_PREFILL_SHARED8) {
+    if (variant == ALICE_PREFILL_SHARED4) { if (d == 64) GOL(2, 4); else if (d == 128) GOL(4, 4); else GOL(8, 4); }
+    else { if (d == 64) GOL(2, 8); else if (d == 128) GOL(4, 8); else GOL(8, 8); }
+    ALICE_LAUNCH_CHECK();
+    return 0;
+  }
   const bool split = variant == ALICE_PREFILL_SPLIT || (variant == ALICE_PREFILL_AUTO && waves2 < 4096);
   if (split) {
     ALICE_CHECK(nH <= 65535, "attention: too many heads for one launch");
@@ -553,6 +724,7 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
     else if (d == 128) { if (gh == 2) GO(4, 2); else GO(4, 1); }
     else { if (gh == 2) GO(8, 2); else GO(8, 1); }
   }
+#undef GOL
 #undef GOS
 #undef GO
   ALICE_LAUNCH_CHECK();

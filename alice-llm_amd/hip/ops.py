@@ -393,14 +393,15 @@ def decode_splits(n_seqs: int, num_kv_heads: int, max_context: int) -> int:
     return max(1, min(by_fill, by_work, 64))
 
 
-PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT = 0, 1, 2
+PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT, PREFILL_SHARED4, PREFILL_SHARED8 = 0, 1, 2, 3, 4
 
 
 def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_table, *, num_heads: int, n_seqs: int,
                       max_new: int, max_context: int, scale: float, softcap: Optional[float], window: Optional[int],
                       variant: int = PREFILL_AUTO) -> None:
-    """Prompt attention on the matrix cores.  variant: whole query tiles per wave, or one tile's keys split over
-    a block's four waves (what fills the chip when there are few tiles); AUTO picks by the grid's size."""
+    """Prompt attention on the matrix cores.  variant: whole query tiles per wave; one tile's keys split over a
+    block's four waves (what fills the chip when there are few tiles); or the four or eight waves of a block
+    sharing each block of keys and values through LDS.  AUTO picks by the grid's size."""
     n_pages, nKV, page_size, d = k_pool.shape
     T = q.shape[0]
     _dev(q, "q", torch.bfloat16, (T, num_heads * d))
