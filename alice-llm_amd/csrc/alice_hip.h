@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 2
+#define ALICE_ABI_VERSION 3
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
@@ -97,8 +97,9 @@ int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool
 int alice_argmax_chunks(int B, int V);
 int alice_argmax(const float* logits, int* out, float* work_v, int* work_i, int B, int V, hipStream_t stream);
 // temperature -> top-k (0: off) -> top-p (>= 1: off) -> softmax -> first index whose cumulative
-// probability exceeds uniform[row].
-int alice_sample(const float* logits, int* out, const float* uniform, int B, int V, float temperature,
+// probability exceeds uniform[row].  work: alice_sample_workspace(B, V) 32-bit words, 8-byte aligned.
+long alice_sample_workspace(int B, int V);
+int alice_sample(const float* logits, int* out, const float* uniform, void* work, int B, int V, float temperature,
                  int top_k, float top_p, hipStream_t stream);
 
 #ifdef __cplusplus

@@ -91,19 +91,26 @@ __device__ __forceinline__ float block_inclusive_scan(float v, float* wred, floa
   return before + v;
 }
 
-// ---- the sampling kernel: one block per row
+// ---- sampling: a row is cut into chunks, a block per chunk for every pass over the row, one block per row
+// for what needs the whole row
 //
-// Every pass over the row is read by the whole block, four consecutive elements per thread per load where the
-// vocabulary is a multiple of four.  The thresholds of top-k and top-p are found among the few largest logits:
-// a pass counts the elements within fixed distances of the maximum, the elements inside the chosen distance
-// (at most CAP) are collected in shared memory, and the first wave bisects the key space over that list.
-// Probabilities enter these comparisons as 64-bit fixed point, so the sums do not depend on the order in
-// which the list was filled.  A row whose kept set does not fit (a flat distribution, a huge k) takes the
-// same bisection over the whole row instead.  The draw goes by index order: sums of tiles of TILE elements
-// (a wave per tile), the tile in which the cumulative sum passes the target, and a scan of that tile alone.
-constexpr int TILE = 4096;       // 4 consecutive elements per thread
+//   chunk_max        the maximum of every chunk
+//   chunk_count      how many elements of the chunk lie within fixed distances of the row's maximum (and, for
+//                    top-p alone, the chunk's probability mass)
+//   chunk_collect    the elements within the chosen distance (at most CAP a row) go to the row's list
+//   row_threshold    the thresholds of top-k and top-p by bisection on the key space over that list, held in
+//                    shared memory; probabilities enter as 64-bit fixed point, so the sums do not depend on the
+//                    order in which the list was filled.  A row whose kept set does not fit (a flat
+//                    distribution, a huge k) takes the same bisection over the whole row instead.
+//   tile_sum         the kept mass of every tile of TILE elements (a wave per tile, lanes in a fixed order)
+//   draw             the tile in which the cumulative sum, in index order, passes the target, and a scan of it
+//
+// Without top-k and top-p only the first and the last two run.  Every pass reads four consecutive elements per
+// thread per load where the vocabulary is a multiple of four.
+constexpr int TILE = 4096;       // 4 consecutive elements per thread of the draw's scan
 constexpr int CAP = 4096;        // candidates held in shared memory
 constexpr int NCUT = 12;
+constexpr int SB = 256;          // threads of the per-chunk kernels
 __device__ constexpr float kCut[NCUT] = {0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f, 8.f, 12.f, 16.f, 24.f, 32.f};
 
 __device__ __forceinline__ float key_value(uint32_t k) {
@@ -127,22 +134,36 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
   return v;
 }
 
-// f(index, logit / T, valid) for every element of the row; every lane of the block runs every call (those past
-// the end with valid = false), in an order that depends on nothing but the thread and V.
-template <int VEC, class F>
-__device__ __forceinline__ void for_row(const float* __restrict__ row, int V, float inv_t, F&& f) {
+// Where a row's intermediate results live (all arrays are per row; `chunks` and `tiles` per row).
+struct SampleWork {
+  float* pmax;                   // [B][chunks]
+  int* pcnt;                     // [B][chunks][NCUT]
+  unsigned long long* pmass;     // [B][chunks]
+  int* ncand;                    // [B]
+  uint32_t* cand;                // [B][CAP]
+  uint32_t* thr;                 // [B]
+  float* tsum;                   // [B][tiles]
+  int* tlast;                    // [B][tiles]
+  int chunks, tiles, tiles_per_chunk;
+};
+
+// f(index, logit / T, valid) for the elements [lo, hi) of a row (lo a multiple of four); every lane of the block
+// runs every call (those past the end with valid = false), in an order that depends on nothing but the thread,
+// the block's size NT and the range.
+template <int VEC, int NT, class F>
+__device__ __forceinline__ void for_range(const float* __restrict__ row, int lo, int hi, float inv_t, F&& f) {
   const int tid = threadIdx.x;
   if constexpr (VEC == 4) {
     constexpr int U = 4;
-    const int G = V >> 2;
+    const int G0 = lo >> 2, G = hi >> 2;
     const float4* r4 = reinterpret_cast<const float4*>(row);
-    for (int g0 = 0; g0 < G; g0 += ST * U) {
+    for (int g0 = G0; g0 < G; g0 += NT * U) {
       float4 x[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) x[u] = r4[min(g0 + u * ST + tid, G - 1)];
+      for (int u = 0; u < U; ++u) x[u] = r4[min(g0 + u * NT + tid, G - 1)];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int g = g0 + u * ST + tid;
+        const int g = g0 + u * NT + tid;
         const bool ok = g < G;
         f(4 * g + 0, x[u].x * inv_t, ok);
         f(4 * g + 1, x[u].y * inv_t, ok);
@@ -152,144 +173,211 @@ __device__ __forceinline__ void for_row(const float* __restrict__ row, int V, fl
     }
   } else {
     constexpr int U = 8;
-    for (int i0 = 0; i0 < V; i0 += ST * U) {
+    for (int i0 = lo; i0 < hi; i0 += NT * U) {
       float x[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) x[u] = row[min(i0 + u * ST + tid, V - 1)];
+      for (int u = 0; u < U; ++u) x[u] = row[min(i0 + u * NT + tid, hi - 1)];
 #pragma unroll
-      for (int u = 0; u < U; ++u) f(i0 + u * ST + tid, x[u] * inv_t, i0 + u * ST + tid < V);
+      for (int u = 0; u < U; ++u) f(i0 + u * NT + tid, x[u] * inv_t, i0 + u * NT + tid < hi);
     }
   }
 }
 
+// The row's maximum from its chunks' (every wave computes it for itself).
+__device__ __forceinline__ float row_max(const SampleWork& w, int b) {
+  float m = -INFINITY;
+  for (int c = threadIdx.x & 63; c < w.chunks; c += 64) m = fmaxf(m, w.pmax[(size_t)b * w.chunks + c]);
+  return wave_max(m);
+}
+
 template <int VEC>
-__global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ logits, int* __restrict__ out,
-                                                    const float* __restrict__ uniform, int V, float inv_t,
-                                                    int top_k, float top_p) {
+__global__ __launch_bounds__(SB) void chunk_max_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t) {
+  __shared__ float red[17];
+  const int b = blockIdx.y, c = blockIdx.x;
+  const float* row = logits + (size_t)b * V;
+  const int lo = c * w.tiles_per_chunk * TILE, hi = min(V, lo + w.tiles_per_chunk * TILE);
+  float lmax = -INFINITY;
+  for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) { lmax = fmaxf(lmax, ok ? x : -INFINITY); });
+  const float m = block_max(lmax, red);
+  if (threadIdx.x == 0) {
+    w.pmax[(size_t)b * w.chunks + c] = m;
+    if (c == 0) w.ncand[b] = 0;
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(SB) void chunk_count_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
+                                                         int whole_mass) {
+  __shared__ int wave_cnt[SB / 64][NCUT];
+  __shared__ unsigned long long wave_mass[SB / 64];
+  const int b = blockIdx.y, c = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float* row = logits + (size_t)b * V;
+  const int lo = c * w.tiles_per_chunk * TILE, hi = min(V, lo + w.tiles_per_chunk * TILE);
+  const float m = row_max(w, b);
+  int cnt[NCUT];
+#pragma unroll
+  for (int j = 0; j < NCUT; ++j) cnt[j] = 0;
+  unsigned long long mass = 0;
+  for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) {
+    const float d = ok ? m - x : INFINITY;
+#pragma unroll
+    for (int j = 0; j < NCUT; ++j) cnt[j] += d <= kCut[j];
+    if (whole_mass && ok) mass += fixed_mass(x, m);
+  });
+  if (whole_mass) mass = wave_sum_u64(mass);
+#pragma unroll
+  for (int j = 0; j < NCUT; ++j) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cnt[j] += __shfl_xor(cnt[j], o, 64);
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int j = 0; j < NCUT; ++j) wave_cnt[wave][j] = cnt[j];
+    wave_mass[wave] = mass;
+  }
+  __syncthreads();
+  if (threadIdx.x < NCUT) {
+    int t = 0;
+    for (int v = 0; v < SB / 64; ++v) t += wave_cnt[v][threadIdx.x];
+    w.pcnt[((size_t)b * w.chunks + c) * NCUT + threadIdx.x] = t;
+  }
+  if (threadIdx.x == 0) {
+    unsigned long long t = 0;
+    for (int v = 0; v < SB / 64; ++v) t += wave_mass[v];
+    w.pmass[(size_t)b * w.chunks + c] = t;
+  }
+}
+
+// The row's counts per distance (and its mass) from the chunks', into tot[NCUT] and *z in shared memory; then the
+// distance whose elements become the list: for top-k the nearest that holds k, else the widest that fits; -1 if
+// none does.  All threads of the block call it (blockDim.x >= 192) and get the same answer.
+__device__ __forceinline__ int choose_cut(const SampleWork& w, int b, bool need_k, int top_k, int* tot, unsigned long long* z) {
+  const int t = threadIdx.x;
+  if (t < NCUT * 16) {
+    const int j = t / 16, part = t % 16;
+    int sum = 0;
+    for (int c = part; c < w.chunks; c += 16) sum += w.pcnt[((size_t)b * w.chunks + c) * NCUT + j];
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    if (part == 0) tot[j] = sum;
+  }
+  if (t == NCUT * 16) {
+    unsigned long long sum = 0;
+    for (int c = 0; c < w.chunks; ++c) sum += w.pmass[(size_t)b * w.chunks + c];
+    *z = sum;
+  }
+  __syncthreads();
+  int cut = -1;
+#pragma unroll
+  for (int j = 0; j < NCUT; ++j) {
+    const int c = tot[j];
+    if (need_k) { if (cut == -1 && c >= top_k && c <= CAP) cut = j; if (cut == -1 && c > CAP) cut = -2; }
+    else if (c >= 1 && c <= CAP) cut = j;
+  }
+  return cut;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(SB) void chunk_collect_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
+                                                           int top_k) {
+  __shared__ int tot[NCUT];
+  __shared__ unsigned long long z;
+  const int b = blockIdx.y, c = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const bool need_k = top_k > 0 && top_k < V;
+  const int cut = choose_cut(w, b, need_k, top_k, tot, &z);
+  if (cut < 0) return;
+  const float* row = logits + (size_t)b * V;
+  const int lo = c * w.tiles_per_chunk * TILE, hi = min(V, lo + w.tiles_per_chunk * TILE);
+  const float m = row_max(w, b);
+  float dcut = kCut[0];
+#pragma unroll
+  for (int j = 0; j < NCUT; ++j) if (j == cut) dcut = kCut[j];
+  uint32_t* list = w.cand + (size_t)b * CAP;
+  for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) {
+    const bool in = ok && (m - x <= dcut);
+    const unsigned long long mask = __ballot(in);
+    if (mask) {
+      const int leader = __ffsll((long long)mask) - 1;
+      int base = 0;
+      if (lane == leader) base = atomicAdd(&w.ncand[b], __popcll(mask));
+      base = __shfl(base, leader, 64);
+      const int pos = base + __popcll(mask & ((1ull << lane) - 1ull));
+      if (in && pos < CAP) list[pos] = order_key(x);
+    }
+  });
+}
+
+template <int VEC>
+__global__ __launch_bounds__(ST) void row_threshold_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
+                                                           int top_k, float top_p) {
   __shared__ float red[17];
   __shared__ int ired[ST / 64];
-  __shared__ float wred[ST / 64];
-  __shared__ float tile_sum[256];                         // sums of up to 256 tiles at a time
-  __shared__ int pick[2];
-  __shared__ float carry[2];
   __shared__ uint32_t list[CAP];
   __shared__ unsigned long long list_mass[CAP];
-  __shared__ int wave_cnt[ST / 64][NCUT];
-  __shared__ unsigned long long wave_mass[ST / 64];
-  __shared__ int n_list;
+  __shared__ int tot[NCUT];
+  __shared__ unsigned long long z_sh;
   __shared__ uint32_t found[3];                           // threshold, top-k done, top-p done
-  const float* row = logits + (size_t)blockIdx.x * V;
+  const int b = blockIdx.x;
+  const float* row = logits + (size_t)b * V;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-  float lmax = -INFINITY;
-  for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) { lmax = fmaxf(lmax, ok ? x : -INFINITY); });
-  const float m = block_max(lmax, red);
+  const float m = row_max(w, b);
   const uint32_t key_m = order_key(m);
-
   const bool need_k = top_k > 0 && top_k < V, need_p = top_p < 1.f;
   uint32_t thr = 0;
   bool k_done = !need_k, p_done = !need_p;
-  if (need_k || need_p) {
-    // how many elements lie within each distance of the maximum (and, for top-p alone, the whole mass)
-    int cnt[NCUT];
-#pragma unroll
-    for (int j = 0; j < NCUT; ++j) cnt[j] = 0;
-    unsigned long long mass = 0;
-    const bool whole_mass = !need_k;
-    for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) {
-      const float d = ok ? m - x : INFINITY;
-#pragma unroll
-      for (int j = 0; j < NCUT; ++j) cnt[j] += d <= kCut[j];
-      if (whole_mass && ok) mass += fixed_mass(x, m);
-    });
-    if (whole_mass) mass = wave_sum_u64(mass);
-#pragma unroll
-    for (int j = 0; j < NCUT; ++j) {
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) cnt[j] += __shfl_xor(cnt[j], o, 64);
-    }
-    if (lane == 0) {
-#pragma unroll
-      for (int j = 0; j < NCUT; ++j) wave_cnt[wave][j] = cnt[j];
-      wave_mass[wave] = mass;
-    }
-    if (tid == 0) { n_list = 0; found[0] = 0; found[1] = 0; found[2] = 0; }
+  if (tid == 0) { found[0] = 0; found[1] = 0; found[2] = 0; }
+  const int cut = choose_cut(w, b, need_k, top_k, tot, &z_sh);
+  if (cut >= 0) {
+    const int n = min(w.ncand[b], CAP);
+    for (int j = tid; j < n; j += ST) list[j] = w.cand[(size_t)b * CAP + j];
     __syncthreads();
-    int cut = -1;                                         // top-k: the nearest distance that holds k; else the widest that fits
-    unsigned long long z_row = 0;
-    {
-      for (int w = 0; w < ST / 64; ++w) z_row += wave_mass[w];
+    if (wave == 0) {
+      const unsigned long long z_row = z_sh;
+      uint32_t kmin = 0xffffffffu;
+      for (int j = lane; j < n; j += 64) kmin = min(kmin, list[j]);
 #pragma unroll
-      for (int j = 0; j < NCUT; ++j) {
-        int c = 0;
-        for (int w = 0; w < ST / 64; ++w) c += wave_cnt[w][j];
-        if (need_k) { if (cut < 0 && c >= top_k && c <= CAP) cut = j; if (cut < 0 && c > CAP) cut = -2; }
-        else if (c >= 1 && c <= CAP) cut = j;
-      }
-    }
-    if (cut >= 0) {
-      float dcut = kCut[0];
-#pragma unroll
-      for (int j = 0; j < NCUT; ++j) if (j == cut) dcut = kCut[j];
-      for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) {
-        const bool c = ok && (m - x <= dcut);
-        const unsigned long long mask = __ballot(c);
-        if (mask) {
-          const int leader = __ffsll((long long)mask) - 1;
-          int base = 0;
-          if (lane == leader) base = atomicAdd(&n_list, __popcll(mask));
-          base = __shfl(base, leader, 64);
-          const int pos = base + __popcll(mask & ((1ull << lane) - 1ull));
-          if (c && pos < CAP) list[pos] = order_key(x);
+      for (int o = 32; o > 0; o >>= 1) kmin = min(kmin, (uint32_t)__shfl_xor(kmin, o, 64));
+      uint32_t t = kmin;
+      if (need_k) {
+        uint32_t lo = kmin, hi = key_m;                   // count(list >= lo) = n >= k
+        while (lo < hi) {
+          const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
+          int c = 0;
+          for (int j0 = 0; j0 < n; j0 += 64) c += __popcll(__ballot(j0 + lane < n && list[min(j0 + lane, n - 1)] >= mid));
+          if (c >= top_k) lo = mid; else hi = mid - 1;
         }
-      });
-      __syncthreads();
-      if (wave == 0) {
-        const int n = min(n_list, CAP);
-        uint32_t kmin = 0xffffffffu;
-        for (int j = lane; j < n; j += 64) kmin = min(kmin, list[j]);
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) kmin = min(kmin, (uint32_t)__shfl_xor(kmin, o, 64));
-        uint32_t t = kmin;
-        if (need_k) {
-          uint32_t lo = kmin, hi = key_m;                 // count(list >= lo) = n >= k
+        t = lo;
+      }
+      bool p_ok = !need_p;
+      if (need_p) {
+        unsigned long long kept = 0;
+        for (int j = lane; j < n; j += 64) {
+          const unsigned long long mass = fixed_mass(key_value(list[j]), m);
+          list_mass[j] = mass;
+          if (list[j] >= t) kept += mass;
+        }
+        kept = wave_sum_u64(kept);                        // the mass of the list at and above the threshold so far
+        const unsigned long long z = need_k ? kept : z_row;
+        const unsigned long long target = (unsigned long long)((double)top_p * (double)z);
+        if (kept > target) {                              // else the nucleus reaches below the list
+          uint32_t lo = t, hi = key_m;
           while (lo < hi) {
             const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
-            int c = 0;
-            for (int j0 = 0; j0 < n; j0 += 64) c += __popcll(__ballot(j0 + lane < n && list[min(j0 + lane, n - 1)] >= mid));
-            if (c >= top_k) lo = mid; else hi = mid - 1;
+            unsigned long long sum = 0;
+            for (int j = lane; j < n; j += 64) if (list[j] >= mid) sum += list_mass[j];
+            sum = wave_sum_u64(sum);
+            if (sum > target) lo = mid; else hi = mid - 1;
           }
           t = lo;
+          p_ok = true;
         }
-        bool p_ok = !need_p;
-        if (need_p) {
-          unsigned long long kept = 0;
-          for (int j = lane; j < n; j += 64) {
-            const unsigned long long w = fixed_mass(key_value(list[j]), m);
-            list_mass[j] = w;
-            if (list[j] >= t) kept += w;
-          }
-          kept = wave_sum_u64(kept);                      // the mass of the list at and above the threshold so far
-          const unsigned long long z = need_k ? kept : z_row;
-          const unsigned long long target = (unsigned long long)((double)top_p * (double)z);
-          if (kept > target) {                            // else the nucleus reaches below the list
-            uint32_t lo = t, hi = key_m;
-            while (lo < hi) {
-              const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
-              unsigned long long sum = 0;
-              for (int j = lane; j < n; j += 64) if (list[j] >= mid) sum += list_mass[j];
-              sum = wave_sum_u64(sum);
-              if (sum > target) lo = mid; else hi = mid - 1;
-            }
-            t = lo;
-            p_ok = true;
-          }
-        }
-        if (lane == 0) { found[0] = t; found[1] = 1; found[2] = p_ok; }
       }
-      __syncthreads();
-      if (found[1]) { k_done = true; if (found[2]) { p_done = true; thr = found[0]; } else if (need_k) thr = found[0]; }
+      if (lane == 0) { found[0] = t; found[1] = 1; found[2] = p_ok; }
     }
+    __syncthreads();
+    if (found[1]) { k_done = true; if (found[2]) { p_done = true; thr = found[0]; } else if (need_k) thr = found[0]; }
   }
   // ---- the same over the whole row, for what the list could not settle
   if (!k_done) {
@@ -297,35 +385,41 @@ __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ lo
     while (lo < hi) {
       const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
       int c = 0;
-      for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) { c += ok && order_key(x) >= mid; });
+      for_range<VEC, ST>(row, 0, V, inv_t, [&](int, float x, bool ok) { c += ok && order_key(x) >= mid; });
       if (block_count(c, ired) >= top_k) lo = mid; else hi = mid - 1;
     }
     thr = lo;
   }
   if (!p_done) {
     float z = 0.f;
-    for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) { if (ok && order_key(x) >= thr) z += expf(x - m); });
+    for_range<VEC, ST>(row, 0, V, inv_t, [&](int, float x, bool ok) { if (ok && order_key(x) >= thr) z += expf(x - m); });
     const float target = top_p * block_sum(z, red);
     uint32_t lo = thr, hi = key_m;
     while (lo < hi) {
       const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
       float s = 0.f;
-      for_row<VEC>(row, V, inv_t, [&](int, float x, bool ok) { if (ok && order_key(x) >= mid) s += expf(x - m); });
+      for_range<VEC, ST>(row, 0, V, inv_t, [&](int, float x, bool ok) { if (ok && order_key(x) >= mid) s += expf(x - m); });
       if (block_sum(s, red) > target) lo = mid; else hi = mid - 1;
     }
     thr = lo;
   }
+  if (tid == 0) w.thr[b] = thr;
+}
 
-  // ---- inverse CDF in index order
-  // pass 1: the kept mass of every tile (wave w takes tiles w, w + 16, ...; lanes in a fixed order), and the
-  // last index with a positive probability
-  const int n_tiles = (V + TILE - 1) / TILE;
-  int last_kept = -1;
-  if (tid == 0) { pick[0] = -1; pick[1] = -1; carry[0] = 0.f; carry[1] = 0.f; }
-  __syncthreads();
-  const float u = uniform[blockIdx.x];
-  auto tile_mass = [&](int t) {
+// The kept mass of every tile of the chunk (wave v takes the chunk's tiles v, v + 4, ...), and the last index with
+// a positive probability in it (-1: none).
+template <int VEC>
+__global__ __launch_bounds__(SB) void tile_sum_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
+                                                      int filtered) {
+  const int b = blockIdx.y, c = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float* row = logits + (size_t)b * V;
+  const float m = row_max(w, b);
+  const uint32_t thr = filtered ? w.thr[b] : 0u;
+  const int t_end = min(w.tiles, (c + 1) * w.tiles_per_chunk);
+  for (int t = c * w.tiles_per_chunk + wave; t < t_end; t += SB / 64) {
     float s = 0.f;
+    int last_kept = -1;
     const int base = t * TILE;
     auto take = [&](int i, float x) {
       if (order_key(x) >= thr) {
@@ -346,51 +440,72 @@ __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ lo
     } else {
       for (int i = base + lane; i < min(V, base + TILE); i += 64) take(i, row[i] * inv_t);
     }
-    return wave_sum(s);
-  };
-  // Two sweeps over the tiles in groups of 256: the first finds the total, the second the tile of the target;
-  // a row of one group keeps its tile sums and needs no second sweep.
+    s = wave_sum(s);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) last_kept = max(last_kept, __shfl_xor(last_kept, o, 64));
+    if (lane == 0) {
+      w.tsum[(size_t)b * w.tiles + t] = s;
+      w.tlast[(size_t)b * w.tiles + t] = last_kept;
+    }
+  }
+}
+
+// Inverse CDF in index order: the running sums of the tiles (one thread, in order), the tile in which the sum
+// passes u times the total, and a scan of that tile, four consecutive elements per thread.
+__global__ __launch_bounds__(ST) void draw_kernel(const float* __restrict__ logits, int* __restrict__ out,
+                                                  const float* __restrict__ uniform, SampleWork w, int V, float inv_t,
+                                                  int filtered) {
+  __shared__ float wred[ST / 64];
+  __shared__ float prefix[1024];                          // inclusive running sums of up to 1024 tiles at a time
+  __shared__ int pick[2];
+  __shared__ float carry[2];
+  const int b = blockIdx.x;
+  const float* row = logits + (size_t)b * V;
+  const int tid = threadIdx.x;
+  const float m = row_max(w, b);
+  const uint32_t thr = filtered ? w.thr[b] : 0u;
+  const float u = uniform[b];
+  const float* tsum = w.tsum + (size_t)b * w.tiles;
+  int last_kept = -1;
+  for (int t = tid; t < w.tiles; t += ST) last_kept = max(last_kept, w.tlast[(size_t)b * w.tiles + t]);
+  if (tid == 0) { pick[0] = -1; pick[1] = -1; carry[0] = 0.f; carry[1] = 0.f; }
+  __syncthreads();
+  atomicMax(&pick[1], last_kept);
+  // the total first (groups of 1024 tiles), then the tile of the target
   for (int sweep = 0; sweep < 2; ++sweep) {
-    const float target = sweep == 1 ? u * carry[0] : 0.f;
-    const bool choose = sweep == 1 || n_tiles <= 256;
+    const float target = u * carry[0];
     float before_group = 0.f;
-    for (int t0 = 0; t0 < n_tiles; t0 += 256) {
-      const int t1 = min(n_tiles, t0 + 256);
-      for (int t = t0 + wave; t < t1; t += ST / 64) {
-        const float s = tile_mass(t);
-        if (lane == 0) tile_sum[t - t0] = s;
-      }
+    for (int t0 = 0; t0 < w.tiles; t0 += 1024) {
+      const int n = min(w.tiles - t0, 1024);
+      __syncthreads();
+      for (int t = tid; t < n; t += ST) prefix[t] = tsum[t0 + t];
       __syncthreads();
       if (tid == 0) {
         float acc = before_group;
-        for (int t = t0; t < t1; ++t) acc += tile_sum[t - t0];
+        for (int t = 0; t < n; ++t) { acc += prefix[t]; prefix[t] = acc; }
         if (sweep == 0) carry[0] = acc;
-        if (choose) {
-          const float tgt = sweep == 1 ? target : u * acc;
-          float run = before_group;
-          for (int t = t0; t < t1; ++t) {
-            const float next = run + tile_sum[t - t0];
-            if (pick[0] < 0 && tgt < next) { pick[0] = t; carry[1] = run; }
-            run = next;
-          }
-        }
-        before_group = acc;
       }
       __syncthreads();
+      if (sweep == 1 || w.tiles <= 1024) {
+        const float tgt = sweep == 1 ? target : u * carry[0];
+        for (int t = tid; t < n; t += ST) {
+          const float lo = t == 0 ? before_group : prefix[t - 1];
+          if (tgt >= lo && tgt < prefix[t]) { pick[0] = t0 + t; carry[1] = lo; }   // at most one tile
+        }
+      }
+      before_group = prefix[n - 1];
     }
-    if (choose) break;
+    if (w.tiles <= 1024) break;
   }
-  atomicMax(&pick[1], last_kept);
   __syncthreads();
   const int t_sel = pick[0], last_of_row = pick[1];
   const float target = u * carry[0];
   const float tile_before = carry[1];
   __syncthreads();
   if (t_sel < 0) {                                       // u * total rounded up to the total: the last kept token
-    if (tid == 0) out[blockIdx.x] = max(last_of_row, 0);
+    if (tid == 0) out[b] = max(last_of_row, 0);
     return;
   }
-  // pass 2: the chosen tile, four consecutive elements per thread, block scan in index order
   if (tid == 0) { pick[0] = -1; pick[1] = -1; }
   const int base = t_sel * TILE + tid * 4;
   float e[4], mine = 0.f;
@@ -412,19 +527,27 @@ __global__ __launch_bounds__(ST) void sample_kernel(const float* __restrict__ lo
   if (target >= before && target < incl) {               // at most one thread: `before` is the thread before's `incl`
     float acc = before;
     int c = my_last;                                     // if rounding lets the run end early: its last positive one
-    bool found = false;
+    bool hit = false;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (!found && e[j] > 0.f) {
+      if (!hit && e[j] > 0.f) {
         acc += e[j];
-        if (target < acc) { c = base + j; found = true; }
+        if (target < acc) { c = base + j; hit = true; }
       }
     }
     pick[0] = c;
   }
   __syncthreads();
   // the tile's sum by waves and by the scan can differ in the last bit: past the scan's end means the tile's last
-  if (tid == 0) out[blockIdx.x] = pick[0] >= 0 ? pick[0] : max(pick[1], 0);
+  if (tid == 0) out[b] = pick[0] >= 0 ? pick[0] : max(pick[1], 0);
+}
+
+// chunks, tiles and tiles per chunk of a call
+__host__ inline void sample_shape(int B, int V, int* chunks, int* tiles, int* per) {
+  *tiles = (V + TILE - 1) / TILE;
+  *per = ((long)B * *tiles + 1023) / 1024;
+  if (*per < 1) *per = 1;
+  *chunks = (*tiles + *per - 1) / *per;
 }
 
 }  // namespace
@@ -454,16 +577,52 @@ extern "C" int alice_argmax(const float* logits, int* out, float* work_v, int* w
   return 0;
 }
 
-extern "C" int alice_sample(const float* logits, int* out, const float* uniform, int B, int V, float temperature,
-                            int top_k, float top_p, hipStream_t stream) {
+// Number of 32-bit words of workspace a call needs.
+extern "C" long alice_sample_workspace(int B, int V) {
+  int chunks, tiles, per;
+  sample_shape(B > 0 ? B : 1, V, &chunks, &tiles, &per);
+  const long rows = B > 0 ? B : 1;
+  // pmass first (8-byte elements), then the 4-byte arrays
+  return rows * chunks * 2 + rows * chunks + rows * chunks * NCUT + rows + rows * CAP + rows + rows * tiles * 2 + 16;
+}
+
+extern "C" int alice_sample(const float* logits, int* out, const float* uniform, void* work, int B, int V,
+                            float temperature, int top_k, float top_p, hipStream_t stream) {
   ALICE_CHECK(B >= 0 && V >= 1, "sample: bad sizes B=%d V=%d", B, V);
   ALICE_CHECK(temperature > 0.f, "sample: temperature must be positive (use argmax for greedy)");
   ALICE_CHECK(top_k >= 0 && top_p > 0.f, "sample: top_k must not be negative and top_p must be positive");
+  ALICE_CHECK(B <= 65535, "sample: %d rows are more than one launch takes", B);
+  ALICE_CHECK(work != nullptr && ((uintptr_t)work & 7) == 0, "sample: the workspace is missing or not 8-byte aligned");
   if (B == 0) return 0;
-  if (V % 4 == 0 && ((uintptr_t)logits & 15) == 0)
-    sample_kernel<4><<<B, ST, 0, stream>>>(logits, out, uniform, V, 1.f / temperature, top_k, top_p);
-  else
-    sample_kernel<1><<<B, ST, 0, stream>>>(logits, out, uniform, V, 1.f / temperature, top_k, top_p);
+  SampleWork w;
+  sample_shape(B, V, &w.chunks, &w.tiles, &w.tiles_per_chunk);
+  const size_t rows = (size_t)B;
+  w.pmass = (unsigned long long*)work;
+  w.pmax = (float*)(w.pmass + rows * w.chunks);
+  w.pcnt = (int*)(w.pmax + rows * w.chunks);
+  w.ncand = w.pcnt + rows * w.chunks * NCUT;
+  w.cand = (uint32_t*)(w.ncand + rows);
+  w.thr = w.cand + rows * CAP;
+  w.tsum = (float*)(w.thr + rows);
+  w.tlast = (int*)(w.tsum + rows * w.tiles);
+  const float inv_t = 1.f / temperature;
+  const bool need_k = top_k > 0 && top_k < V, need_p = top_p < 1.f;
+  const int filtered = need_k || need_p;
+  const dim3 cgrid(w.chunks, B);
+#define GO(VEC)                                                                                                             \
+  do {                                                                                                                      \
+    chunk_max_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t);                                                   \
+    if (filtered) {                                                                                                         \
+      chunk_count_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, need_k ? 0 : 1);                               \
+      chunk_collect_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, top_k);                                      \
+      row_threshold_kernel<VEC><<<B, ST, 0, stream>>>(logits, w, V, inv_t, top_k, top_p);                                   \
+    }                                                                                                                       \
+    tile_sum_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, filtered);                                          \
+  } while (0)
+  if (V % 4 == 0 && ((uintptr_t)logits & 15) == 0) GO(4); else GO(1);
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  draw_kernel<<<B, ST, 0, stream>>>(logits, out, uniform, w, V, inv_t, filtered);
   ALICE_LAUNCH_CHECK();
   return 0;
 }

@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA = 0, 1, 2, 3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 _lock = threading.Lock()
@@ -50,7 +50,8 @@ def _declare(lib) -> None:
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
         "alice_argmax_chunks": [I, I],
-        "alice_sample": [P, P, P, I, I, F, I, F, P],
+        "alice_sample_workspace": [I, I],
+        "alice_sample": [P, P, P, P, I, I, F, I, F, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -488,6 +489,9 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     return out
 
 
+_sample_work = {}        # (device, B, V) -> the workspace of sample(): calls on one device's stream follow each other
+
+
 def sample(logits: torch.Tensor, uniform: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0,
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """int32 [B]: temperature, top-k, top-p, softmax and inverse CDF with uniform[row] in [0, 1)."""
@@ -497,6 +501,13 @@ def sample(logits: torch.Tensor, uniform: torch.Tensor, temperature: float, top_
     if out is None:
         out = torch.empty((B,), dtype=torch.int32, device=logits.device)
     _dev(out, "out", torch.int32, (B,))
-    _call("alice_sample", logits.data_ptr(), out.data_ptr(), uniform.data_ptr(), B, V, float(temperature),
-          int(top_k), float(top_p), _stream())
+    key = (logits.device, B, V)
+    work = _sample_work.get(key)
+    if work is None:
+        if len(_sample_work) > 16:
+            _sample_work.clear()
+        work = _sample_work[key] = torch.empty((library().alice_sample_workspace(B, V) + 1) // 2, dtype=torch.int64,
+                                               device=logits.device)
+    _call("alice_sample", logits.data_ptr(), out.data_ptr(), uniform.data_ptr(), work.data_ptr(), B, V,
+          float(temperature), int(top_k), float(top_p), _stream())
     return out
