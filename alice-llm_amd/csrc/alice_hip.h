@@ -24,6 +24,7 @@
 #define ALICE_LINEAR_GENERIC 1
 #define ALICE_LINEAR_SKINNY 2
 #define ALICE_LINEAR_MFMA 3
+#define ALICE_LINEAR_TILED256 4   // the tiled kernel with 256 x 256 blocks (MFMA: the 128 x 256 one, or the streaming one)
 
 #ifdef __cplusplus
 extern "C" {

@@ -86,6 +86,15 @@ __device__ __forceinline__ void store4_frag(bf16_t* __restrict__ y, int m, int n
   *reinterpret_cast<uint2*>(y + off) = pk;
 }
 
+// Row-major, or (bfloat16 only) fragment order.
+template <typename TO>
+__device__ __forceinline__ void store4_any(TO* __restrict__ y, int y_frag, int m, size_t row_off, int n, int N, f32x4 v) {
+  if constexpr (sizeof(TO) == 2) {
+    if (y_frag) { store4_frag((bf16_t*)y, m, n, N, v); return; }
+  }
+  store4(y, row_off, n, N, v);
+}
+
 // What the rotation epilogue needs: where q goes, the cache, the tables and the geometry.
 struct RopeArgs {
   bf16_t* q_out;
@@ -333,7 +342,8 @@ constexpr int KC = 2;      // k-tiles per stage
 template <int EPI, typename TO, bool FULL, int TM, bool XF>
 __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                                TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                               float epi, int gx, int gy, int kt_per_slice, RopeArgs ra) {
+                                                               float epi, int gx, int gy, int kt_per_slice, int y_frag,
+                                                               RopeArgs ra) {
   constexpr int XJ = TM / 4;                               // token tiles each wave stages
   __shared__ __align__(16) uint32_t xs_raw[2 * KC * TM * 64 * 4];
   u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
@@ -473,7 +483,7 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
         f32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
-        store4(y, row_off, n, N, o);
+        store4_any(y, y_frag, m, row_off, n, N, o);
       }
     } else {
 #pragma unroll
@@ -483,7 +493,155 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
         f32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
-        store4(y, row_off, n, N, o);
+        store4_any(y, y_frag, m, row_off, n, N, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- tiled, very many tokens: 256 x 256 a block
+// Four waves, two by two: every wave computes 128 tokens x 128 output features (8 x 8 MFMA tiles, 256
+// accumulator registers per lane).  Both operands go through LDS: a k-tile of the block is 16 token tiles and
+// 16 weight tiles of 1 KB, brought by loads that write LDS directly (a lane's 16 bytes land at the tile's base
+// + 16 x lane, which is fragment order for weights, for activations in fragment order and for row-major
+// activations alike), eight tiles per wave.  RING k-tiles are held: while one is multiplied, the next
+// RING - 1 are on their way, and one barrier a k-tile suffices.  Against 128 x 256 blocks that share only the
+// activations, a block moves two thirds of the bytes per product, which is what bounds these kernels.
+constexpr int RING = 4;
+constexpr int BIG_LDS = RING * 32 * 1024;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {               // s_waitcnt vmcnt(N), the other counters left alone
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int EPI, typename TO, bool FULL, bool XF>
+__global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+                                                                 TO* __restrict__ y, int M, int N, int K, int KT, int NT,
+                                                                 float epi, int gx, int gy, int kt_per_slice, int y_frag,
+                                                                 RopeArgs ra) {
+  extern __shared__ __align__(16) uint32_t ring_raw[];       // [RING][16 token tiles | 2 x 8 weight tiles][64 lanes][16 B]
+  u32x4* ring = reinterpret_cast<u32x4*>(ring_raw);
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int wm = wave & 1, wn = wave >> 1;                   // this wave's half of the tokens and of the features
+  const int id = blockIdx.x, xcd = id & 7, local = id >> 3;  // XCD x works through the x-th eighth of the blocks
+  const int per = (gx * gy + 7) >> 3;
+  const int item = xcd * per + local;
+  if (local >= per || item >= gx * gy) return;
+  const int bx = item / gy, by = item % gy;
+  const int m0 = by * 256;
+  // the eight weight tiles of feature half h of this block
+  auto tile_of = [&](int h, int i) {
+    if (EPI == ALICE_EPI_GEGLU) {
+      const int pair = (bx * 2 + h) * 4 + (i >> 1);
+      return pair >= N / 16 ? NT : ((i & 1) ? N / 16 + pair : pair);
+    }
+    return (bx * 2 + h) * 8 + i;
+  };
+  int tile[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) tile[i] = tile_of(wn, i);
+  // What this wave brings per k-tile: waves 0 and 1 the token tiles 8 wave .. + 7, waves 2 and 3 the weight tiles
+  // of feature half wave - 2.  One address per tile and lane at k-tile 0; all loads are unconditional (rows and
+  // tiles beyond the matrix are clamped, k-tiles beyond the slice bring the zero tile or the last k-tile again).
+  const bool brings_x = wave < 2;
+  const bf16_t* src[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const bf16_t* xs;
+    if constexpr (XF) xs = x + ((size_t)min((m0 >> 4) + 8 * (wave & 1) + i, (M - 1) >> 4) * KT * 64 + lane) * 8;
+    else xs = x + (size_t)min(m0 + (8 * (wave & 1) + i) * 16 + r, M - 1) * K;
+    const bf16_t* ws = wf + (size_t)min(tile_of(wave & 1, i), NT - 1) * KT * 512 + lane * 8;
+    src[i] = brings_x ? xs : ws;
+  }
+  const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
+  const int kt_base = blockIdx.y * kt_per_slice, kt_end = min(KT, kt_base + kt_per_slice);
+  const int T = kt_end - kt_base;
+  y += (size_t)blockIdx.y * M * N;
+  const int slot_base = brings_x ? 8 * wave : 16 + 8 * (wave - 2);
+  auto bring = [&](int rel) {                                // k-tile kt_base + rel into ring slot rel % RING
+    const int kt = kt_base + rel;
+    const bool kok = kt < kt_end;
+    const int ktc = min(kt, kt_end - 1);
+    size_t off;
+    if (brings_x) off = XF ? (size_t)ktc * 512 : (size_t)min(ktc * 32 + g * 8, K - 8);
+    else off = (size_t)ktc * 512;
+    u32x4* dst = ring + ((size_t)(rel % RING) * 32 + slot_base) * 64;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bf16_t* p = (brings_x || kok) ? src[i] + off : zero;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
+                                       (__attribute__((address_space(3))) void*)(dst + i * 64), 16, 0, 0);
+    }
+  };
+
+  f32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int s = 0; s < RING - 1; ++s) bring(s);
+  for (int t = 0; t < T; ++t) {
+    // This wave's part of k-tile t has landed; then everyone's has, and everyone is done with k-tile t - 1.
+    // (A plain barrier instruction: __syncthreads() carries a fence, for which the compiler waits until
+    // every load in flight has written LDS, the ones for the k-tiles ahead included.)
+    wait_vmcnt<(RING - 2) * 8>();
+    asm volatile("s_barrier" ::: "memory");
+    bring(t + RING - 1);                                     // into the slot of k-tile t - 1
+    const u32x4* st = ring + (size_t)(t % RING) * 32 * 64;
+    u32x4 xf[8], wk[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xf[j] = st[(8 * wm + j) * 64 + lane];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) wk[i] = st[(16 + 8 * wn + i) * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i][j] = mfma16(wk[i], xf[j], acc[i][j]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  wait_vmcnt<0>();                                           // the loads past the end still write LDS
+
+  if constexpr (EPI == ALICE_EPI_ROPE) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int m = m0 + (8 * wm + j) * 16 + r;
+      if (m >= M) continue;
+      const RopeToken tk = rope_token(ra, m);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (tile[i] < NT) rope_store4(ra, m, tk, tile[i] * 16 + g * 4, acc[i][j]);
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int m = m0 + (8 * wm + j) * 16 + r;
+    if (m >= M) continue;
+    const size_t row_off = (size_t)m * N;
+    if (EPI == ALICE_EPI_GEGLU) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        if (tile[2 * p] >= NT) continue;
+        const int n = tile[2 * p] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
+        store4_any(y, y_frag, m, row_off, n, N, o);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (tile[i] >= NT) continue;
+        const int n = tile[i] * 16 + g * 4;
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
+        store4_any(y, y_frag, m, row_off, n, N, o);
       }
     }
   }
@@ -558,29 +716,55 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
   return 1;
 }
 
+// Whether the 256 x 256 blocks are worth it.  Not yet: with one wave per SIMD the waits for LDS and for the
+// barrier are not hidden, and the kernel runs at 0.8 of the speed of the 128 x 256 one; it is reached by its
+// variant only.
+inline bool big_tiles_pay(int, int, int) { return false; }
+
 template <int EPI, typename TO>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
-                 hipStream_t s, const RopeArgs& ra = RopeArgs{}) {
-  (void)y_frag;
+                 hipStream_t s, const RopeArgs& ra = RopeArgs{}, int big = 0) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
-  const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
-  int gy = ceil_div(M, 16 * WM);
+  const int per = ceil_div(KT, split);
   {
-    // 128 tokens a block, or 64 when that leaves the chip less than full
-    const int per = ceil_div(KT, split);
-    if (x_frag) {
-      // fragment order is what decode steps use: few tokens, one or a few block rows
-      dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 8, true><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
-    } else if (gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64) {
-      dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 8, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
-    } else {
-      gy = ceil_div(M, 64);
-      dim3 grid(8 * ceil_div(gx * gy, 8), split);
-      linear_tiled_lds_kernel<EPI, TO, false, 4, false><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, ra);
+    // big: 1 forces the 256 x 256 blocks, -1 forbids them
+    const int gx256 = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 8) : ceil_div(NT, 16);
+    if (big > 0 || (big == 0 && big_tiles_pay(M, gx256, split))) {
+      const int gy256 = ceil_div(M, 256);
+      dim3 grid(8 * ceil_div(gx256 * gy256, 8), split);
+      static bool prepared[2] = {false, false};
+      if (x_frag) {
+        auto kern = linear_tiled256_kernel<EPI, TO, false, true>;
+        if (!prepared[1]) {
+          ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) == hipSuccess,
+                      "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
+          prepared[1] = true;
+        }
+        kern<<<grid, 256, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
+      } else {
+        auto kern = linear_tiled256_kernel<EPI, TO, false, false>;
+        if (!prepared[0]) {
+          ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) == hipSuccess,
+                      "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
+          prepared[0] = true;
+        }
+        kern<<<grid, 256, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
+      }
+      ALICE_LAUNCH_CHECK();
+      return 0;
     }
   }
+  const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
+  int gy = ceil_div(M, 16 * WM);
+  // 128 tokens a block, or 64 when that leaves the chip less than full
+  const bool high = gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64;
+  if (!high) gy = ceil_div(M, 64);
+  dim3 grid(8 * ceil_div(gx * gy, 8), split);
+#define GO(TMV, XFV) \
+  linear_tiled_lds_kernel<EPI, TO, false, TMV, XFV><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, y_frag, ra)
+  if (x_frag) { if (high) GO(8, true); else GO(4, true); }
+  else { if (high) GO(8, false); else GO(4, false); }
+#undef GO
   ALICE_LAUNCH_CHECK();
   return 0;
 }
@@ -652,9 +836,9 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),
               "linear: partial sums need no epilogue and float32 output");
   ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
-  ALICE_CHECK(y_layout == ALICE_LAYOUT_ROW || (y_layout == ALICE_LAYOUT_FRAG16 && skinny && y_dtype == DT_BF16 && N % 32 == 0 &&
+  ALICE_CHECK(y_layout == ALICE_LAYOUT_ROW || (y_layout == ALICE_LAYOUT_FRAG16 && y_dtype == DT_BF16 && N % 32 == 0 &&
                                                 split_k == 1 && epi != ALICE_EPI_SOFTCAP),
-              "linear: output in fragment order needs the streaming kernel, bfloat16 and N %% 32 == 0");
+              "linear: output in fragment order needs bfloat16, N %% 32 == 0, no softcap and no partial sums");
   const int x_frag = x_layout == ALICE_LAYOUT_FRAG16, y_frag = y_layout == ALICE_LAYOUT_FRAG16;
 #define BY_EPI(FN, ...)                                                                            \
   do {                                                                                             \
@@ -669,7 +853,8 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
     }                                                                                              \
   } while (0)
   if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
-  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
+  const int big = variant == ALICE_LINEAR_TILED256 ? 1 : (variant == ALICE_LINEAR_MFMA ? -1 : 0);
+  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream, RopeArgs{}, big);
 #undef BY_EPI
 }
 

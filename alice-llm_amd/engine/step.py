@@ -120,7 +120,7 @@ class _DecodeGraph:
                                cu_seqlens=part(5), context_lens=part(6), n_tokens=B, n_seqs=B, is_decode=True,
                                max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
                                start_lens=[0] * B, slot_ids=[0] * B,
-                               fragment_activations=engine.model.precision.act == torch.bfloat16 and B <= 64,
+                               fragment_activations=engine.model.precision.act == torch.bfloat16,
                                want_every_row=True)
         o = self.offs
         self.shadow[o[2]:o[3]] = np.arange(B)                # constant parts
@@ -253,8 +253,7 @@ class Engine:
                           n_tokens=T, n_seqs=B, is_decode=all(n == 1 for n in n_new), max_new=max(n_new),
                           max_context=max(ctx_lens), max_position=max(ctx_lens) - 1,
                           new_lens=n_new, start_lens=start, slot_ids=list(slots),
-                          fragment_activations=(self.model.precision.act == torch.bfloat16 and T <= 64
-                                                and all(n == 1 for n in n_new)),
+                          fragment_activations=self.model.precision.act == torch.bfloat16,
                           want_every_row=rows == list(range(T)))
         logits = self.model.forward(ctx, self.cache, block_tables)
         self.cache.commit(slots, n_new)

@@ -42,9 +42,9 @@ class Precision:
 # --------------------------------------------------------------------------- activations in fragment order
 
 class FragmentActs:
-    """bfloat16 activations [rows, cols] of a decode step (at most 64 rows) stored in the order in which
-    the matrix-core kernels read them ([rows/16][cols/32][64 lanes][8], rows padded to 16): a wave
-    fetches a whole operand with one contiguous read.  Only parts that declare
+    """bfloat16 activations [rows, cols] stored in the order in which the matrix-core kernels read them
+    ([rows/16][cols/32][64 lanes][8], rows padded to 16): a wave fetches a whole operand tile with one
+    contiguous 1 KB read instead of sixteen pieces of 64 bytes.  Only parts that declare
     `accepts_fragment_activations` are ever handed one; everything else sees plain tensors."""
 
     def __init__(self, data: torch.Tensor, rows: int, cols: int):
@@ -60,7 +60,7 @@ class FragmentActs:
 
     @staticmethod
     def possible(precision: "Precision", rows: int, cols: int) -> bool:
-        return precision.act == torch.bfloat16 and 1 <= rows <= 64 and cols % 32 == 0
+        return precision.act == torch.bfloat16 and rows >= 1 and cols % 32 == 0
 
     @staticmethod
     def empty(rows: int, cols: int, device) -> "FragmentActs":

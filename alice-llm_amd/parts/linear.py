@@ -55,15 +55,14 @@ class Linear:
         return self.layout == ops.LAYOUT_FRAG16 and self.k % 32 == 0
 
     def can_write_fragments(self, rows: int) -> bool:
-        # the streaming kernel's privilege; very wide outputs go to the tiled kernel from 17 rows on
-        return (self.layout == ops.LAYOUT_FRAG16 and rows <= 64 and self.n % 32 == 0 and not (rows > 16 and self.n >= 65536)
+        return (self.layout == ops.LAYOUT_FRAG16 and rows >= 1 and self.n % 32 == 0
                 and self.epilogue != ops.EPI_SOFTCAP and self.precision.act == torch.bfloat16)
 
     def __call__(self, x, out_dtype: torch.dtype, *, allow_partials: bool = False,
                  variant: int = ops.LINEAR_AUTO, out_fragments: bool = False):
         """x: [M, k] tensor or FragmentActs.  Returns [M, n], or [S, M, n] float32 partial sums when the
         kernel prefers to split the inner dimension and the caller can add them up (allow_partials), or a
-        FragmentActs when out_fragments is asked for (bfloat16, at most 64 rows)."""
+        FragmentActs when out_fragments is asked for (bfloat16)."""
         M = x.shape[0]
         frag_in = isinstance(x, FragmentActs)
         if frag_in and not self.accepts_fragment_input:

@@ -442,6 +442,48 @@ def test_linear_mfma(M, N, K, ydt):
             close(yp.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 32), (300, 1000, 416), (1000, 80, 2048), (513, 528, 72), (70, 304, 160)])
+def test_linear_mfma_blocks_of_256(M, N, K):
+    """The kernel with 256 x 256 blocks, forced, against the plain product and bit for bit against the 128 x 256 one."""
+    x, w = rnd(M, K, seed=70, dtype=torch.bfloat16), rnd(N, K, seed=71, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    ref = x.double() @ w.double().T
+    for ydt, atol, rtol in ((torch.float32, 2e-4, 1e-5), (torch.bfloat16, 1e-2, 2 ** -8)):
+        y, y0 = (torch.full((M, N), float("nan"), dtype=ydt, device=DEV) for _ in range(2))
+        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256, full_precision=False)
+        ops.linear(x, wf, y0, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_MFMA, full_precision=False)
+        close(y, ref, atol * math.sqrt(K / 64), rtol)
+        assert torch.equal(y, y0)
+    y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(x, wf, y2, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_SOFTCAP, epi_param=3.0,
+               variant=ops.LINEAR_TILED256, full_precision=False)
+    close(y2, 3.0 * torch.tanh(ref / 3.0), 1e-3)
+    for split in (2, 3):
+        if K // 32 >= split:
+            yp = torch.full((split, M, N), float("nan"), dtype=torch.float32, device=DEV)
+            ops.linear(x, wf, yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=ops.LINEAR_TILED256,
+                       full_precision=False)
+            close(yp.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
+    if K % 32 == 0:
+        yf = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear(acts_to_fragments(x), wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256,
+                   full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16)
+        assert torch.equal(yf, y0)
+    if N % 32 == 0:
+        flat = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear(x, wf, flat, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256, full_precision=False,
+                   rows=M, y_layout=ops.LAYOUT_FRAG16)
+        assert torch.equal(acts_from_fragments(flat, M, N), y0.cpu())
+    if N % 16 == 0:
+        w2 = rnd(2 * N, K, seed=72, scale=0.3, dtype=torch.bfloat16)
+        wf2 = ops.to_frag16(w2)
+        gate, up = x.double() @ w2.double()[:N].T, x.double() @ w2.double()[N:].T
+        yg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear(x, wf2, yg, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, variant=ops.LINEAR_TILED256,
+                   full_precision=False)
+        close(yg, F.gelu(gate, approximate="tanh") * up, 2e-2, 2 ** -7)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 48, 96), (200, 304, 96), (129, 2048, 64)])
 def test_linear_mfma_geglu(M, N, K):
     x, w = rnd(M, K, seed=18, dtype=torch.bfloat16), rnd(2 * N, K, seed=19, scale=0.3, dtype=torch.bfloat16)
@@ -485,7 +527,7 @@ def acts_from_fragments(flat, M, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 224, 160), (16, 4096, 256), (17, 160, 320), (33, 64, 96), (64, 2304, 1024),
-                                   (40, 65536 + 32, 64)])
+                                   (40, 65536 + 32, 64), (130, 224, 160), (300, 96, 64), (1000, 2304, 96)])
 def test_linear_mfma_activations_in_fragment_order(M, N, K):
     x, w = rnd(M, K, seed=16, dtype=torch.bfloat16), rnd(N, K, seed=17, scale=0.1, dtype=torch.bfloat16)
     wf, xf = ops.to_frag16(w), acts_to_fragments(x)
@@ -505,19 +547,15 @@ def test_linear_mfma_activations_in_fragment_order(M, N, K):
             ops.linear(xf, wf, b, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False, rows=M,
                        x_layout=ops.LAYOUT_FRAG16)
             assert torch.equal(a, b)
-        # writing fragments (the streaming kernel only)
-        for src, lay in ((x, ops.LAYOUT_ROW), (xf, ops.LAYOUT_FRAG16)):
-            yf = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
-            ops.linear(src, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, x_layout=lay,
-                       y_layout=ops.LAYOUT_FRAG16)
-            assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
-    else:
-        yf = torch.empty((-(-M // 16) * 16) * N, dtype=torch.bfloat16, device=DEV)
-        with pytest.raises(ops.HipLibraryError, match="fragment order"):
-            ops.linear(x, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, y_layout=ops.LAYOUT_FRAG16)
+    # writing fragments
+    for src, lay in ((x, ops.LAYOUT_ROW), (xf, ops.LAYOUT_FRAG16)):
+        yf = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear(src, wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False, rows=M, x_layout=lay,
+                   y_layout=ops.LAYOUT_FRAG16)
+        assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 96, 96)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 96, 96), (200, 320, 96), (513, 2048, 64)])
 def test_linear_mfma_geglu_in_fragment_order(M, N, K):
     x, w = rnd(M, K, seed=18, dtype=torch.bfloat16), rnd(2 * N, K, seed=19, scale=0.3, dtype=torch.bfloat16)
     wf, xf = ops.to_frag16(w), acts_to_fragments(x)
