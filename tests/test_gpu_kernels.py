@@ -444,7 +444,8 @@ def test_linear_mfma(M, N, K, ydt):
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (300, 1000, 416), (1000, 80, 2048), (513, 528, 72), (70, 304, 160)])
 def test_linear_mfma_blocks_of_256(M, N, K):
-    """The kernel with 256 x 256 blocks, forced, against the plain product and bit for bit against the 128 x 256 one."""
+    """The kernel with 256 x 256 blocks, forced, against the plain product (its MFMA adds 16 inner elements at a
+    time, the other kernels' 32: the same sums in another order)."""
     x, w = rnd(M, K, seed=70, dtype=torch.bfloat16), rnd(N, K, seed=71, scale=0.1, dtype=torch.bfloat16)
     wf = ops.to_frag16(w)
     ref = x.double() @ w.double().T
@@ -453,7 +454,7 @@ def test_linear_mfma_blocks_of_256(M, N, K):
         ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256, full_precision=False)
         ops.linear(x, wf, y0, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_MFMA, full_precision=False)
         close(y, ref, atol * math.sqrt(K / 64), rtol)
-        assert torch.equal(y, y0)
+        close(y0, ref, atol * math.sqrt(K / 64), rtol)
     y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
     ops.linear(x, wf, y2, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_SOFTCAP, epi_param=3.0,
                variant=ops.LINEAR_TILED256, full_precision=False)
@@ -468,12 +469,12 @@ def test_linear_mfma_blocks_of_256(M, N, K):
         yf = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
         ops.linear(acts_to_fragments(x), wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256,
                    full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16)
-        assert torch.equal(yf, y0)
+        assert torch.equal(yf, y)                          # the same bits from rows and from fragments
     if N % 32 == 0:
         flat = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
         ops.linear(x, wf, flat, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED256, full_precision=False,
                    rows=M, y_layout=ops.LAYOUT_FRAG16)
-        assert torch.equal(acts_from_fragments(flat, M, N), y0.cpu())
+        assert torch.equal(acts_from_fragments(flat, M, N), y.cpu())
     if N % 16 == 0:
         w2 = rnd(2 * N, K, seed=72, scale=0.3, dtype=torch.bfloat16)
         wf2 = ops.to_frag16(w2)
