@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 3
+#define ALICE_ABI_VERSION 4
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
@@ -87,7 +87,7 @@ int alice_attention_mfma_supported(int d);
 int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
                             const int* cu_seqlens, const int* context_lens, const int* block_table,
                             int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
-                            float scale, float softcap, int window, int variant, hipStream_t stream);
+                            float scale, float softcap, int window, int variant, int out_layout, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                            const int* context_lens, const int* block_table, int bt_stride, int B, int nH,

@@ -220,6 +220,14 @@ struct Core {
   }
 };
 
+// Where output element (token or sequence b, column c of nH * D) goes: row-major, or fragment order for the
+// output projection ([rows/16][nH*D/32][64][8]; four consecutive columns from a multiple of four are neighbours
+// in both).
+__device__ __forceinline__ size_t decode_out_index(int layout, int b, int c, int width) {
+  if (layout == 0) return (size_t)b * width + c;
+  return ((size_t)((size_t)(b >> 4) * (width >> 5) + (c >> 5)) * 64 + ((c & 31) >> 3) * 16 + (b & 15)) * 8 + (c & 7);
+}
+
 // ---------------------------------------------------------------- prompts
 // grid: (tiles of 64 query tokens, sequences, kv heads x passes); 4 waves, wave w takes tokens
 // 16 w .. 16 w + 15 of the tile for GH query heads of one kv head (a pass); the passes of a kv head's
@@ -231,7 +239,8 @@ template <int DT, int GH, bool SOFTCAP>
 __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
-    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window,
+    int out_layout) {
   constexpr int D = DT * 32;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
@@ -303,12 +312,11 @@ __global__ __launch_bounds__(256, GH == 1 ? 2 : 1) void attn_prefill_kernel(
     if (pos[hh] < 0) continue;
     const int head = kvh * group + h0 + hh;
     const float inv = 1.f / c.l[hh];
-    bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
 #pragma unroll
     for (int t = 0; t < 2 * DT; ++t) {
       const f32x4 v = c.o[hh][t] * inv;
       uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
-      *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+      *reinterpret_cast<uint2*>(out + decode_out_index(out_layout, t_begin + my_tok, head * D + t * 16 + g * 4, nH * D)) = pk;
     }
   }
 }
@@ -322,7 +330,8 @@ template <int DT, bool SOFTCAP>
 __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
-    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window) {
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window,
+    int out_layout) {
   constexpr int D = DT * 32;
   __shared__ float sm[4][16], sl[4][16];
   extern __shared__ __align__(16) float so[];                // [3 waves][16 columns][D + 4]
@@ -391,7 +400,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
     ll += sl[w][col] * f[w];
   }
   const float inv = 1.f / ll;
-  bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + head) * D;
 #pragma unroll
   for (int t = 0; t < 2 * DT; ++t) {
     f32x4 v = c.o[0][t] * f[0];
@@ -400,7 +408,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
       v += *reinterpret_cast<const f32x4*>(&so[((size_t)(w - 1) * 16 + col) * (D + 4) + t * 16 + g * 4]) * f[w];
     v *= inv;
     uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
-    *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+    *reinterpret_cast<uint2*>(out + decode_out_index(out_layout, t_begin + my_tok, head * D + t * 16 + g * 4, nH * D)) = pk;
   }
 }
 
@@ -415,7 +423,8 @@ template <int DT, bool SOFTCAP, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
-    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int HB) {
+    const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int HB,
+    int out_layout) {
   constexpr int D = DT * 32;
   constexpr int NT = 64 * NW;
   constexpr int PIECES = 4 * DT * 64;                        // 16-byte pieces of a block: keys, then values
@@ -493,20 +502,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_
   c.finish();
   if (!tok_ok) return;
   const float inv = 1.f / c.l[0];
-  bf16_t* orow = out + ((size_t)(t_begin + my_tok) * nH + kvh * group + hh) * D;
 #pragma unroll
   for (int t = 0; t < 2 * DT; ++t) {
     const f32x4 v = c.o[0][t] * inv;
     uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
-    *reinterpret_cast<uint2*>(orow + t * 16 + g * 4) = pk;
+    *reinterpret_cast<uint2*>(out + decode_out_index(out_layout, t_begin + my_tok, (kvh * group + hh) * D + t * 16 + g * 4, nH * D)) = pk;
   }
-}
-
-// Where output element (sequence b, column c of nH * D) goes: row-major, or fragment order for the output
-// projection's streaming kernel ([B/16][nH*D/32][64][8]).
-__device__ __forceinline__ size_t decode_out_index(int layout, int b, int c, int width) {
-  if (layout == 0) return (size_t)b * width + c;
-  return ((size_t)((size_t)(b >> 4) * (width >> 5) + (c >> 5)) * 64 + ((c & 31) >> 3) * 16 + (b & 15)) * 8 + (c & 7);
 }
 
 // ---------------------------------------------------------------- single tokens, keys split over blocks
@@ -651,8 +652,9 @@ extern "C" int alice_attention_mfma_supported(int d) { return d == 64 || d == 12
 extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
                                        const int* cu_seqlens, const int* context_lens, const int* block_table,
                                        int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
-                                       float scale, float softcap, int window, int variant, hipStream_t stream) {
+                                       float scale, float softcap, int window, int variant, int out_layout, hipStream_t stream) {
   ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
+  ALICE_CHECK(out_layout == 0 || (out_layout == 1 && (nH * d) % 32 == 0), "attention: unknown output layout %d", out_layout);
   ALICE_CHECK(nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
   ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
   ALICE_CHECK(B >= 0 && max_new >= 0 && B <= 65535 && nKV <= 65535, "attention: bad batch B=%d", B);
@@ -669,10 +671,10 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   do {                                                                                                                      \
     if (softcap > 0.f)                                                                                                      \
       attn_prefill_kernel<DT, GH, true><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, out_layout);     \
     else                                                                                                                    \
       attn_prefill_kernel<DT, GH, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, out_layout);     \
   } while (0)
 #define GOS(DT)                                                                                                             \
   do {                                                                                                                      \
@@ -680,10 +682,10 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
     const size_t lds = (size_t)3 * 16 * (DT * 32 + 4) * sizeof(float);                                                      \
     if (softcap > 0.f)                                                                                                      \
       attn_prefill_split_kernel<DT, true><<<sgrid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, out_layout);     \
     else                                                                                                                    \
       attn_prefill_split_kernel<DT, false><<<sgrid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window);                 \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, out_layout);     \
   } while (0)
   // Few waves (one prompt of a few thousand tokens): split every tile's keys over four waves.  Many: whole
   // tiles per wave, two heads a wave where the group is even.
@@ -695,10 +697,10 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
     const size_t lds = (size_t)2 * 4 * DT * 1024;                                                                           \
     if (softcap > 0.f)                                                                                                      \
       attn_prefill_shared_kernel<DT, true, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb);             \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb, out_layout); \
     else                                                                                                                    \
       attn_prefill_shared_kernel<DT, false, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb);             \
+          (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb, out_layout); \
   } while (0)
   // Which form (measured on Gemma 2 shapes): with many blocks, four waves sharing their keys; with fewer, eight
   // (half as many blocks, half the key traffic); with too few blocks to fill the chip, one tile's keys split

@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED256 = 0, 1, 2, 3, 4
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 _lock = threading.Lock()
@@ -45,7 +45,7 @@ def _declare(lib) -> None:
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, P],
         "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
-        "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
+        "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -399,14 +399,18 @@ PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT, PREFILL_SHARED4, PREFILL_SHARED8 = 0
 
 def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_table, *, num_heads: int, n_seqs: int,
                       max_new: int, max_context: int, scale: float, softcap: Optional[float], window: Optional[int],
-                      variant: int = PREFILL_AUTO) -> None:
+                      variant: int = PREFILL_AUTO, out_layout: int = LAYOUT_ROW) -> None:
     """Prompt attention on the matrix cores.  variant: whole query tiles per wave; one tile's keys split over a
     block's four waves (what fills the chip when there are few tiles); or the four or eight waves of a block
-    sharing each block of keys and values through LDS.  AUTO picks by the grid's size."""
+    sharing each block of keys and values through LDS.  AUTO picks by the grid's size.
+    out_layout FRAG16: `out` is a flat buffer of ceil16(T) * num_heads * d elements in fragment order."""
     n_pages, nKV, page_size, d = k_pool.shape
     T = q.shape[0]
     _dev(q, "q", torch.bfloat16, (T, num_heads * d))
-    _dev(out, "out", torch.bfloat16, (T, num_heads * d))
+    if out_layout == LAYOUT_FRAG16:
+        _dev(out, "out", torch.bfloat16, (frag_rows(T) * num_heads * d,))
+    else:
+        _dev(out, "out", torch.bfloat16, (T, num_heads * d))
     _dev(k_pool, "k_pool", torch.bfloat16)
     _dev(v_pool, "v_pool", torch.bfloat16, k_pool.shape)
     _dev(cu_seqlens, "cu_seqlens", torch.int32, (n_seqs + 1,))
@@ -417,7 +421,7 @@ def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_ta
     _call("alice_attention_prefill", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
           cu_seqlens.data_ptr(), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_seqs,
           max_new, num_heads, nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), int(variant),
-          _stream())
+          int(out_layout), _stream())
 
 
 def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,
@@ -452,7 +456,7 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
               out_layout: int = LAYOUT_ROW) -> None:
     """Attention of the step's query tokens over the cache; picks the kernel for the step's shape and
     the cache's layout.  `ctx` carries positions, seq_of_token, cu_seqlens, context_lens and the
-    host-side sizes of the step.  out_layout FRAG16 is taken by the single-token kernel only."""
+    host-side sizes of the step.  out_layout FRAG16 is taken by the matrix-core kernels only."""
     if kv_layout == KV_FRAGMENT:
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
@@ -460,14 +464,13 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
                              max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
                              out_layout=out_layout)
             return
-        if out_layout != LAYOUT_ROW:
-            raise HipLibraryError("only the single-token attention kernel writes fragment order")
         attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
                           num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
-                          max_context=ctx.max_context, scale=scale, softcap=softcap, window=window)
+                          max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
+                          out_layout=out_layout)
         return
     if out_layout != LAYOUT_ROW:
-        raise HipLibraryError("only the single-token attention kernel writes fragment order")
+        raise HipLibraryError("only the matrix-core attention kernels write fragment order")
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
                       max_position=ctx.max_position, full_precision=full_precision)

@@ -95,10 +95,9 @@ class Attention(Part):
                 self.position.rotate_and_store(qkv, q, ctx, cache, pair_order=True, **geometry)
             else:
                 self.position.rotate_and_store(qkv, q, ctx, cache, **geometry)
-        # Single tokens on the matrix-core kernel: its output goes to the output projection in fragment order.
-        frag = (getattr(ctx, "fragment_activations", False) and ctx.is_decode and self.kv_layout == ops.KV_FRAGMENT
-                and self.nH // self.nKV <= 16 and self.o.accepts_fragment_input
-                and FragmentActs.possible(self.precision, T, self.q_dim))
+        # The matrix-core kernels' output goes to the output projection in fragment order.
+        frag = (getattr(ctx, "fragment_activations", False) and self.kv_layout == ops.KV_FRAGMENT
+                and self.o.accepts_fragment_input and FragmentActs.possible(self.precision, T, self.q_dim))
         out = FragmentActs.empty(T, self.q_dim, q.device) if frag else torch.empty_like(q)
         ops.attention(q, cache.k, cache.v, out.data if frag else out, ctx, cache.block_table, num_heads=self.nH,
                       scale=self.scale, softcap=self.softcap, window=self.window, full_precision=self.precision.full,

@@ -782,6 +782,14 @@ def test_attention_mfma_prompts(nH, nKV, d, cap, window):
             ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
                                   max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant)
             close(out, ref, 2e-2)
+            if (nH * d) % 32 == 0 and variant != ops.PREFILL_AUTO:
+                # output in fragment order for the projection that follows: the same bits, elsewhere
+                T = q.shape[0]
+                flat = torch.full(((-(-T // 16) * 16) * nH * d,), float("nan"), dtype=torch.bfloat16, device=DEV)
+                ops.attention_prefill(q, kp, vp, flat, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
+                                      max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant,
+                                      out_layout=ops.LAYOUT_FRAG16)
+                assert torch.equal(acts_from_fragments(flat, T, nH * d), out.cpu())
 
 
 @pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
