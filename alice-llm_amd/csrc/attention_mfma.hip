@@ -15,6 +15,7 @@
 // S[key 4(l/16) + i][query l%16]; two such tiles, rounded to bfloat16, are exactly the second operand
 // of the value product in the key order that the value layout above stores, so the probabilities
 // never move between lanes.  Each lane keeps the running maximum and sum of its query column.
+#include <type_traits>
 #include "common.h"
 #include "alice_hip.h"
 
@@ -32,6 +33,7 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
 
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RAISE = 8.f;   // how far a maximum may outgrow the softmax's exponent base before the base follows
 
 // Constants of the score pipeline.  A raw dot product s becomes, in the base-2 domain in which the
 // softmax runs (2^y = e^score):
@@ -162,20 +164,30 @@ struct Core {
       const int lo = window > 0 ? max(pos[b] + 1 - window, 0) : 0;
       const unsigned span = pos[b] >= 0 ? (unsigned)(pos[b] - lo) : 0u;
       const int rel0 = pos[b] >= 0 ? key0 + g * 4 - lo : 1 << 30;
+      // Most blocks lie wholly inside every query's range: no masking then (a column without a query takes what
+      // comes; nothing of it is ever stored).
+      const bool all_seen = __all(pos[b] < 0 || (key0 >= lo && key0 + 31 <= pos[b]));
       float mx = -INFINITY;
+      auto transform = [&](auto masked) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = s[b][t][i] * k.c_in;
-          if (SOFTCAP) v = fmaf(-2.f * k.c_out, rcp_fast(exp2_fast(v) + 1.f), k.c_out);
-          v = ((unsigned)(rel0 + t * 16 + i) <= span) ? v : -INFINITY;
-          s[b][t][i] = v;
-          mx = fmaxf(mx, v);
-        }
-      const float m_new = fmaxf(m[b], col_max(mx));
+          for (int i = 0; i < 4; ++i) {
+            float v = s[b][t][i] * k.c_in;
+            if (SOFTCAP) v = fmaf(-2.f * k.c_out, rcp_fast(exp2_fast(v) + 1.f), k.c_out);
+            if (decltype(masked)::value) v = ((unsigned)(rel0 + t * 16 + i) <= span) ? v : -INFINITY;
+            s[b][t][i] = v;
+            mx = fmaxf(mx, v);
+          }
+      };
+      if (all_seen) transform(std::false_type{}); else transform(std::true_type{});
+      // The exponent base follows the maximum only when the maximum has outgrown it by more than RAISE (in
+      // base-2 exponent units): probabilities then reach 2^RAISE at most, which float32 sums and bfloat16
+      // operands hold as well as values up to 1, and the output is rescaled in a few blocks instead of in most.
+      const float seen = col_max(mx);
+      const bool raise = seen > m[b] + RAISE;
+      const float m_new = raise ? seen : m[b];
       const float base = (m_new == -INFINITY) ? 0.f : m_new;                    // all masked so far: every p is 0
-      const float corr = exp2_fast(m[b] - base);                                // m[b] = -inf gives 0
       float sum = 0.f;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -185,14 +197,16 @@ struct Core {
           s[b][t][i] = e;
           sum += e;
         }
-      l[b] = l[b] * corr + sum;
-      m[b] = m_new;
       p[b] = u32x4{pack2(s[b][0][0], s[b][0][1]), pack2(s[b][0][2], s[b][0][3]),
                    pack2(s[b][1][0], s[b][1][1]), pack2(s[b][1][2], s[b][1][3])};
-      if (corr != 1.f) {
+      if (__any(raise)) {                                                       // the whole wave or none of it
+        const float corr = raise ? exp2_fast(m[b] - base) : 1.f;               // m[b] = -inf gives 0
+        l[b] *= corr;
 #pragma unroll
         for (int t = 0; t < 2 * DT; ++t) o[b][t] *= corr;
       }
+      l[b] += sum;
+      m[b] = m_new;
     }
   }
 
