@@ -19,6 +19,7 @@
 #define ALICE_PREFILL_SPLIT 2   // the four waves of a block split one tile's keys
 #define ALICE_PREFILL_SHARED4 3 // the four waves of a block share each block of keys and values through LDS
 #define ALICE_PREFILL_SHARED8 4 // the same with eight waves
+#define ALICE_PREFILL_SHARED4X2 5 // two sets of four waves, each with half of the block's keys
 
 #define ALICE_LINEAR_AUTO 0
 #define ALICE_LINEAR_GENERIC 1

@@ -433,19 +433,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_split_kernel(
 // the next block is on its way from memory into registers while this one is computed, and one barrier a
 // step suffices.  Against whole tiles per wave, memory traffic falls by the number of waves.
 // grid: (tiles of 16 NW / HB tokens, from the end backwards; sequences; kv heads x passes over the group).
-template <int DT, bool SOFTCAP, int NW>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_kernel(
+template <int DT, bool SOFTCAP, int NW, int KS>
+__global__ __launch_bounds__(64 * NW * KS, NW * KS == 4 ? 2 : 1) void attn_prefill_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     bf16_t* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
     const int* __restrict__ block_table, int bt_stride, int nH, int nKV, float scale, float cap, int window, int HB,
     int out_layout) {
+  // KS = 2: two sets of NW waves, the second takes the later half of the block's keys (its own buffers in LDS);
+  // at the end the first set adds the second's part to its own, each scaled to the common maximum.  Halves the
+  // longest block's run when there are too few blocks to fill the chip.
   constexpr int D = DT * 32;
-  constexpr int NT = 64 * NW;
+  constexpr int NT = 64 * NW;                                // threads of a set
   constexpr int PIECES = 4 * DT * 64;                        // 16-byte pieces of a block: keys, then values
   constexpr int CH = (PIECES + NT - 1) / NT;                 // pieces per thread
-  extern __shared__ __align__(16) uint32_t kv_raw[];         // [2 buffers][keys 2 DT KB | values 2 DT KB]
-  u32x4* kv = reinterpret_cast<u32x4*>(kv_raw);
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  extern __shared__ __align__(16) uint32_t kv_raw[];         // [KS sets][2 buffers][keys 2 DT KB | values 2 DT KB]
+  const int lane = threadIdx.x & 63, wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int set = wave_all / NW, wave = wave_all % NW, tid = threadIdx.x % NT;
+  u32x4* kv = reinterpret_cast<u32x4*>(kv_raw) + (size_t)set * 2 * PIECES;
   const int col = lane & 15, g = lane >> 4;
   const int group = nH / nKV, passes = (group + HB - 1) / HB;
   const int b = blockIdx.y, kvh = blockIdx.z / passes, hh = (blockIdx.z % passes) * HB + wave % HB;
@@ -463,11 +467,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_
   const int* bt = block_table + (size_t)b * bt_stride;
   const size_t page_elems = (size_t)64 * D;
   const ScoreConsts sc(scale, cap);
-  // the block's run of key blocks, and this wave's own within it
+  // the block's run of key blocks, this set's part of it, and this wave's own within that
   const int block_last_pos = start_len + min(block_first + tokens, n_new) - 1;
-  const int kb_begin = (window > 0 ? max(0, start_len + block_first + 1 - window) : 0) >> 5, kb_end = block_last_pos >> 5;
-  const int my_begin = (window > 0 ? max(0, start_len + first + 1 - window) : 0) >> 5;
-  const int my_end = wave_ok ? (start_len + min(first + 15, n_new - 1)) >> 5 : -1;
+  const int run_begin = (window > 0 ? max(0, start_len + block_first + 1 - window) : 0) >> 5, run_end = block_last_pos >> 5;
+  const int steps = (run_end - run_begin + KS) / KS;         // of the first set: ceil(blocks / KS)
+  const int kb_begin = run_begin + set * steps, kb_end = min(run_end, kb_begin + steps - 1);
+  const int my_begin = max(kb_begin, (window > 0 ? max(0, start_len + first + 1 - window) : 0) >> 5);
+  const int my_end = wave_ok ? min(kb_end, (start_len + min(first + 15, n_new - 1)) >> 5) : -1;
 
   Core<DT, 1> c;
   c.init();
@@ -479,32 +485,33 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_
       if (tok_ok) c.q[0][dt] = *reinterpret_cast<const u32x4*>(qrow + dt * 32 + g * 8);
     }
   }
-  // piece j of a thread: piece threadIdx.x + NT j of the block.  Loads are unconditional: past the last block
-  // the last one is fetched again, and a piece past the end is the last piece.
+  // piece j of a thread: piece tid + NT j of the block.  Loads are unconditional: past the set's last block
+  // (or, for an empty second set, before its first) a block of the run is fetched again, and a piece past the
+  // end is the last piece.
   u32x4 st[CH];
   auto fetch = [&](int kb32) {
-    kb32 = min(kb32, kb_end);
+    kb32 = min(min(kb32, max(kb_end, kb_begin)), run_end);
     const int page = bt[kb32 >> 1];
     const u32x4* kp = reinterpret_cast<const u32x4*>(k_pool + ((size_t)page * nKV + kvh) * page_elems) + (size_t)(kb32 & 1) * 2 * DT * 64;
     const u32x4* vp = reinterpret_cast<const u32x4*>(v_pool + ((size_t)page * nKV + kvh) * page_elems) + (size_t)(kb32 & 1) * 2 * DT * 64;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int piece = min((int)threadIdx.x + NT * j, PIECES - 1);
+      const int piece = min(tid + NT * j, PIECES - 1);
       st[j] = *(piece < 2 * DT * 64 ? kp + piece : vp + (piece - 2 * DT * 64));
     }
   };
   auto put = [&](int buf) {
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int piece = (int)threadIdx.x + NT * j;
+      const int piece = tid + NT * j;
       if (PIECES % NT == 0 || piece < PIECES) kv[(size_t)buf * PIECES + piece] = st[j];
     }
   };
   fetch(kb_begin);
   put(0);
   __syncthreads();
-  for (int kb32 = kb_begin; kb32 <= kb_end; ++kb32) {
-    const int buf = (kb32 - kb_begin) & 1;
+  for (int it = 0; it < steps; ++it) {                       // both sets take the same number of steps
+    const int kb32 = kb_begin + it, buf = it & 1;
     fetch(kb32 + 1);
     if (kb32 >= my_begin && kb32 <= my_end) {
       const u32x4* kl = kv + (size_t)buf * PIECES;
@@ -514,6 +521,32 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_shared_
     __syncthreads();
   }
   c.finish();
+  if constexpr (KS == 2) {
+    // the second set leaves its part where the key buffers were (everyone is past the last barrier of the loop)
+    float* so = reinterpret_cast<float*>(kv_raw);            // [NW waves][16 columns][D + 4], then maxima and sums
+    float* sm = so + NW * 16 * (D + 4);
+    float* sl = sm + NW * 16;
+    if (set == 1) {
+      if (g == 0) { sm[wave * 16 + col] = c.m[0]; sl[wave * 16 + col] = c.l[0]; }
+#pragma unroll
+      for (int t = 0; t < 2 * DT; ++t)
+        *reinterpret_cast<f32x4*>(&so[((size_t)wave * 16 + col) * (D + 4) + t * 16 + g * 4]) = c.o[0][t];
+    }
+    __syncthreads();
+    if (set == 1 || !tok_ok) return;
+    const float m1 = sm[wave * 16 + col], l1 = sl[wave * 16 + col];
+    const float mm = fmaxf(c.m[0], m1);
+    const float f0 = (c.m[0] == -INFINITY) ? 0.f : exp2_fast(c.m[0] - mm), f1 = (m1 == -INFINITY) ? 0.f : exp2_fast(m1 - mm);
+    const float inv = 1.f / (c.l[0] * f0 + l1 * f1);
+#pragma unroll
+    for (int t = 0; t < 2 * DT; ++t) {
+      f32x4 v = c.o[0][t] * f0 + *reinterpret_cast<const f32x4*>(&so[((size_t)wave * 16 + col) * (D + 4) + t * 16 + g * 4]) * f1;
+      v *= inv;
+      uint2 pk = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+      *reinterpret_cast<uint2*>(out + decode_out_index(out_layout, t_begin + my_tok, (kvh * group + hh) * D + t * 16 + g * 4, nH * D)) = pk;
+    }
+    return;
+  }
   if (!tok_ok) return;
   const float inv = 1.f / c.l[0];
 #pragma unroll
@@ -678,7 +711,7 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   // Two heads a wave halve the key/value reads.
   const long waves2 = (long)ceil_div(max_new, 64) * B * nKV * ceil_div(group, 2) * 4;
   const int gh = group % 2 == 0 ? 2 : 1;
-  ALICE_CHECK(variant >= 0 && variant <= 4, "attention: unknown variant %d", variant);
+  ALICE_CHECK(variant >= 0 && variant <= 5, "attention: unknown variant %d", variant);
   ALICE_CHECK((long)nKV * ceil_div(group, gh) <= 65535, "attention: too many heads for one launch");
   dim3 grid(ceil_div(max_new, 64), B, nKV * ceil_div(group, gh));
 #define GO(DT, GH)                                                                                                          \
@@ -703,31 +736,43 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
   } while (0)
   // Few waves (one prompt of a few thousand tokens): split every tile's keys over four waves.  Many: whole
   // tiles per wave, two heads a wave where the group is even.
-#define GOL(DT, NW)                                                                                                         \
+#define GOL(DT, NW, KS)                                                                                                     \
   do {                                                                                                                      \
     const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);                                                           \
     ALICE_CHECK((long)nKV * ceil_div(group, hb) <= 65535, "attention: too many heads for one launch");                      \
     dim3 lgrid(ceil_div(max_new, 16 * NW / hb), B, nKV * ceil_div(group, hb));                                              \
-    const size_t lds = (size_t)2 * 4 * DT * 1024;                                                                           \
+    const size_t lds = (size_t)KS * 2 * 4 * DT * 1024;                                                                      \
+    static bool prepared = false;                                                                                           \
+    if (lds > 65536 && !prepared) {                                                                                         \
+      ALICE_CHECK(hipFuncSetAttribute((const void*)attn_prefill_shared_kernel<DT, true, NW, KS>,                            \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess &&                \
+                  hipFuncSetAttribute((const void*)attn_prefill_shared_kernel<DT, false, NW, KS>,                           \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess,                  \
+                  "attention: the device does not give a block %d bytes of LDS", (int)lds);                                 \
+      prepared = true;                                                                                                      \
+    }                                                                                                                       \
     if (softcap > 0.f)                                                                                                      \
-      attn_prefill_shared_kernel<DT, true, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+      attn_prefill_shared_kernel<DT, true, NW, KS><<<lgrid, 64 * NW * KS, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
           (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb, out_layout); \
     else                                                                                                                    \
-      attn_prefill_shared_kernel<DT, false, NW><<<lgrid, 64 * NW, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
+      attn_prefill_shared_kernel<DT, false, NW, KS><<<lgrid, 64 * NW * KS, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
           (bf16_t*)out, cu_seqlens, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, hb, out_layout); \
   } while (0)
   // Which form (measured on Gemma 2 shapes): with many blocks, four waves sharing their keys; with fewer, eight
-  // (half as many blocks, half the key traffic); with too few blocks to fill the chip, one tile's keys split
-  // over a block's waves.  Small heads spend their time in the softmax arithmetic and gain nothing from sharing.
+  // (half as many blocks, half the key traffic); with too few blocks to fill the chip, the keys of a block split
+  // over two sets of four waves, or one tile's keys split over a block's waves.  Small heads spend their time in
+  // the softmax arithmetic and gain nothing from sharing.
   if (variant == ALICE_PREFILL_AUTO && d >= 128) {
     const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
     const long per_tile = (long)B * nKV * ceil_div(group, hb);
     if (per_tile * ceil_div(max_new, 64 / hb) >= 2048) variant = ALICE_PREFILL_SHARED4;
     else if (per_tile * ceil_div(max_new, 128 / hb) >= 192) variant = ALICE_PREFILL_SHARED8;
+    else if (per_tile * ceil_div(max_new, 64 / hb) >= 192 && max_new >= 1024) variant = ALICE_PREFILL_SHARED4X2;
   }
-  if (variant == ALICE_PREFILL_SHARED4 || variant == ALICE_PREFILL_SHARED8) {
-    if (variant == ALICE_PREFILL_SHARED4) { if (d == 64) GOL(2, 4); else if (d == 128) GOL(4, 4); else GOL(8, 4); }
-    else { if (d == 64) GOL(2, 8); else if (d == 128) GOL(4, 8); else GOL(8, 8); }
+  if (variant == ALICE_PREFILL_SHARED4 || variant == ALICE_PREFILL_SHARED8 || variant == ALICE_PREFILL_SHARED4X2) {
+    if (variant == ALICE_PREFILL_SHARED4) { if (d == 64) GOL(2, 4, 1); else if (d == 128) GOL(4, 4, 1); else GOL(8, 4, 1); }
+    else if (variant == ALICE_PREFILL_SHARED8) { if (d == 64) GOL(2, 8, 1); else if (d == 128) GOL(4, 8, 1); else GOL(8, 8, 1); }
+    else { if (d == 64) GOL(2, 4, 2); else if (d == 128) GOL(4, 4, 2); else GOL(8, 4, 2); }
     ALICE_LAUNCH_CHECK();
     return 0;
   }

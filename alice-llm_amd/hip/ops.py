@@ -394,7 +394,7 @@ def decode_splits(n_seqs: int, num_kv_heads: int, max_context: int) -> int:
     return max(1, min(by_fill, by_work, 64))
 
 
-PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT, PREFILL_SHARED4, PREFILL_SHARED8 = 0, 1, 2, 3, 4
+PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT, PREFILL_SHARED4, PREFILL_SHARED8, PREFILL_SHARED4X2 = 0, 1, 2, 3, 4, 5
 
 
 def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_table, *, num_heads: int, n_seqs: int,

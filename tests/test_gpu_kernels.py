@@ -777,7 +777,7 @@ def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K,
 def test_attention_mfma_prompts(nH, nKV, d, cap, window):
     for lens, new in (((5, 130, 66), (5, 130, 66)), ((150, 64, 33), (20, 3, 33)), ((300,), (300,))):
         q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, new, cap, window, seed=3)
-        for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_AUTO):
+        for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_SHARED4X2, ops.PREFILL_AUTO):
             out = torch.full_like(q, float("nan"))
             ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
                                   max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant)
@@ -810,7 +810,7 @@ def test_attention_mfma_single_tokens(nH, nKV, d, cap, window):
                              window=window, out_layout=ops.LAYOUT_FRAG16)
         assert torch.equal(acts_from_fragments(flat, len(lens), nH * d), out.cpu())
     # the prompt kernels on single tokens give the same
-    for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8):
+    for variant in (ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_SHARED4X2):
         out = torch.full_like(q, float("nan"))
         ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=1, max_context=max(lens),
                               scale=scale, softcap=cap, window=window, variant=variant)
@@ -823,7 +823,7 @@ def test_attention_mfma_far_key_and_window_edge():
         k[3] = 0; k[3, :, 0] = 40.0
         q[L - 1] = 0; q[L - 1, :, 0] = 40.0
     q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, None, seed=5, crafted=far)
-    for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8):
+    for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_SHARED4X2):
         out = torch.full_like(q, float("nan"))
         if fn == "decode":
             ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=None)
@@ -837,7 +837,7 @@ def test_attention_mfma_far_key_and_window_edge():
             k[where] = 0; k[where, :, 0] = 40.0; v[where] = 7.0
             q[L - 1] = 0; q[L - 1, :, 0] = 40.0
         q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, (L,), (1,), None, 100, seed=6, crafted=edge)
-        for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8):
+        for fn in ("decode", ops.PREFILL_TILES, ops.PREFILL_SPLIT, ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_SHARED4X2):
             out = torch.full_like(q, float("nan"))
             if fn == "decode":
                 ops.attention_decode(q, kp, vp, out, ctx, bt, num_heads=nH, max_context=L, scale=scale, softcap=None, window=100)
