@@ -812,8 +812,10 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
   }
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
-  // 128 tokens a block, or 64 when that leaves the chip less than full
-  const bool high = gx * gy * split >= 384 || (split > 1 && gx * gy * split >= 256) || M <= 64;
+  // 128 tokens a block, or 64 when that leaves most of the chip without a block (measured at N = 2304 and 4096:
+  // 216 and 256 blocks of 128 tokens beat twice as many of 64, 128 blocks do not; with the rotation epilogue,
+  // whose stores are scattered, 256 blocks of 128 tokens lose against 512 of 64)
+  const bool high = gx * gy * split >= (EPI == ALICE_EPI_ROPE ? 384 : 192) || M <= 64;
   if (!high) gy = ceil_div(M, 64);
   dim3 grid(8 * ceil_div(gx * gy, 8), split);
 #define GO(TMV, XFV) \
