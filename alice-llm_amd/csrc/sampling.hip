@@ -97,9 +97,10 @@ __device__ __forceinline__ float block_inclusive_scan(float v, float* wred, floa
 //   chunk_max        the maximum of every chunk
 //   chunk_count      how many elements of the chunk lie within fixed distances of the row's maximum (and, for
 //                    top-p alone, the chunk's probability mass)
-//   chunk_collect    the elements within the chosen distance (at most CAP a row) go to the row's list
+//   chunk_collect    the elements within the chosen distance (at most CAPG a row) go to the row's list
 //   row_threshold    the thresholds of top-k and top-p by bisection on the key space over that list, held in
-//                    shared memory; probabilities enter as 64-bit fixed point, so the sums do not depend on the
+//                    shared memory (up to CAP candidates: one wave does it) or read from memory by the whole
+//                    block; probabilities enter as 64-bit fixed point, so the sums do not depend on the
 //                    order in which the list was filled.  A row whose kept set does not fit (a flat
 //                    distribution, a huge k) takes the same bisection over the whole row instead.
 //   tile_sum         the kept mass of every tile of TILE elements (a wave per tile, lanes in a fixed order)
@@ -109,9 +110,12 @@ __device__ __forceinline__ float block_inclusive_scan(float v, float* wred, floa
 // thread per load where the vocabulary is a multiple of four.
 constexpr int TILE = 4096;       // 4 consecutive elements per thread of the draw's scan
 constexpr int CAP = 4096;        // candidates held in shared memory
+constexpr int CAPG = 32768;      // candidates of a row's list in memory
 constexpr int NCUT = 12;
 constexpr int SB = 256;          // threads of the per-chunk kernels
-__device__ constexpr float kCut[NCUT] = {0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f, 8.f, 12.f, 16.f, 24.f, 32.f};
+constexpr int NMC = 4;           // distances at which the mass inside is summed too (top-p alone)
+__device__ constexpr int kMassCut[NMC] = {5, 7, 8, 9};   // indices into kCut: 4, 8, 10, 12
+__device__ constexpr float kCut[NCUT] = {0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f, 8.f, 10.f, 12.f, 16.f, 24.f};
 
 __device__ __forceinline__ float key_value(uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
@@ -138,9 +142,9 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
 struct SampleWork {
   float* pmax;                   // [B][chunks]
   int* pcnt;                     // [B][chunks][NCUT]
-  unsigned long long* pmass;     // [B][chunks]
-  int* ncand;                    // [B]
-  uint32_t* cand;                // [B][CAP]
+  unsigned long long* pmass;     // [B][chunks][1 + NMC]: the chunk's mass, and its mass within kCut[kMassCut[i]] of the maximum
+  uint32_t* cand;                // [B][CAPG]
+  unsigned long long* cmass;     // [B][CAPG]: the candidates' masses, for lists too long for shared memory
   uint32_t* thr;                 // [B]
   float* tsum;                   // [B][tiles]
   int* tlast;                    // [B][tiles]
@@ -201,7 +205,6 @@ __global__ __launch_bounds__(SB) void chunk_max_kernel(const float* __restrict__
   const float m = block_max(lmax, red);
   if (threadIdx.x == 0) {
     w.pmax[(size_t)b * w.chunks + c] = m;
-    if (c == 0) w.ncand[b] = 0;
   }
 }
 
@@ -209,7 +212,7 @@ template <int VEC>
 __global__ __launch_bounds__(SB) void chunk_count_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
                                                          int whole_mass) {
   __shared__ int wave_cnt[SB / 64][NCUT];
-  __shared__ unsigned long long wave_mass[SB / 64];
+  __shared__ unsigned long long wave_mass[SB / 64][1 + NMC];
   const int b = blockIdx.y, c = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float* row = logits + (size_t)b * V;
@@ -218,14 +221,24 @@ __global__ __launch_bounds__(SB) void chunk_count_kernel(const float* __restrict
   int cnt[NCUT];
 #pragma unroll
   for (int j = 0; j < NCUT; ++j) cnt[j] = 0;
-  unsigned long long mass = 0;
+  unsigned long long mass[1 + NMC];
+#pragma unroll
+  for (int i = 0; i <= NMC; ++i) mass[i] = 0;
   for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) {
     const float d = ok ? m - x : INFINITY;
 #pragma unroll
     for (int j = 0; j < NCUT; ++j) cnt[j] += d <= kCut[j];
-    if (whole_mass && ok) mass += fixed_mass(x, m);
+    if (whole_mass && ok) {
+      const unsigned long long e = fixed_mass(x, m);
+      mass[0] += e;
+#pragma unroll
+      for (int i = 0; i < NMC; ++i) mass[1 + i] += d <= kCut[kMassCut[i]] ? e : 0ull;
+    }
   });
-  if (whole_mass) mass = wave_sum_u64(mass);
+  if (whole_mass) {
+#pragma unroll
+    for (int i = 0; i <= NMC; ++i) mass[i] = wave_sum_u64(mass[i]);
+  }
 #pragma unroll
   for (int j = 0; j < NCUT; ++j) {
 #pragma unroll
@@ -234,7 +247,8 @@ __global__ __launch_bounds__(SB) void chunk_count_kernel(const float* __restrict
   if (lane == 0) {
 #pragma unroll
     for (int j = 0; j < NCUT; ++j) wave_cnt[wave][j] = cnt[j];
-    wave_mass[wave] = mass;
+#pragma unroll
+    for (int i = 0; i <= NMC; ++i) wave_mass[wave][i] = mass[i];
   }
   __syncthreads();
   if (threadIdx.x < NCUT) {
@@ -242,17 +256,20 @@ __global__ __launch_bounds__(SB) void chunk_count_kernel(const float* __restrict
     for (int v = 0; v < SB / 64; ++v) t += wave_cnt[v][threadIdx.x];
     w.pcnt[((size_t)b * w.chunks + c) * NCUT + threadIdx.x] = t;
   }
-  if (threadIdx.x == 0) {
+  if (threadIdx.x < 1 + NMC) {
     unsigned long long t = 0;
-    for (int v = 0; v < SB / 64; ++v) t += wave_mass[v];
-    w.pmass[(size_t)b * w.chunks + c] = t;
+    for (int v = 0; v < SB / 64; ++v) t += wave_mass[v][threadIdx.x];
+    w.pmass[((size_t)b * w.chunks + c) * (1 + NMC) + threadIdx.x] = t;
   }
 }
 
-// The row's counts per distance (and its mass) from the chunks', into tot[NCUT] and *z in shared memory; then the
-// distance whose elements become the list: for top-k the nearest that holds k, else the widest that fits; -1 if
-// none does.  All threads of the block call it (blockDim.x >= 192) and get the same answer.
-__device__ __forceinline__ int choose_cut(const SampleWork& w, int b, bool need_k, int top_k, int* tot, unsigned long long* z) {
+// The row's counts per distance (and, for top-p alone, its mass and the masses within some distances) from the
+// chunks', into tot[NCUT] and z[1 + NMC] in shared memory; then the distance whose elements become the list:
+// for top-k the nearest that holds k; for top-p alone the nearest whose mass clearly exceeds p times the row's,
+// else the widest that fits; -1 if none does.  All threads of the block call it (blockDim.x >= 256) and get the
+// same answer.
+__device__ __forceinline__ int choose_cut(const SampleWork& w, int b, bool need_k, int top_k, float top_p, int* tot,
+                                          unsigned long long* z) {
   const int t = threadIdx.x;
   if (t < NCUT * 16) {
     const int j = t / 16, part = t % 16;
@@ -262,31 +279,40 @@ __device__ __forceinline__ int choose_cut(const SampleWork& w, int b, bool need_
     for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
     if (part == 0) tot[j] = sum;
   }
-  if (t == NCUT * 16) {
+  if (t >= NCUT * 16 && t < NCUT * 16 + 1 + NMC && !need_k) {
     unsigned long long sum = 0;
-    for (int c = 0; c < w.chunks; ++c) sum += w.pmass[(size_t)b * w.chunks + c];
-    *z = sum;
+    for (int c = 0; c < w.chunks; ++c) sum += w.pmass[((size_t)b * w.chunks + c) * (1 + NMC) + (t - NCUT * 16)];
+    z[t - NCUT * 16] = sum;
   }
   __syncthreads();
   int cut = -1;
+  if (!need_k) {
+    const unsigned long long target = (unsigned long long)((double)top_p * (double)z[0]);
+#pragma unroll
+    for (int i = 0; i < NMC; ++i) {
+      const int c = tot[kMassCut[i]];
+      if (cut == -1 && c >= 1 && c <= CAPG && z[1 + i] > target + (target >> 16)) cut = kMassCut[i];
+    }
+    if (cut >= 0) return cut;
+  }
 #pragma unroll
   for (int j = 0; j < NCUT; ++j) {
     const int c = tot[j];
-    if (need_k) { if (cut == -1 && c >= top_k && c <= CAP) cut = j; if (cut == -1 && c > CAP) cut = -2; }
-    else if (c >= 1 && c <= CAP) cut = j;
+    if (need_k) { if (cut == -1 && c >= top_k && c <= CAPG) cut = j; if (cut == -1 && c > CAPG) cut = -2; }
+    else if (c >= 1 && c <= CAPG) cut = j;
   }
   return cut;
 }
 
 template <int VEC>
 __global__ __launch_bounds__(SB) void chunk_collect_kernel(const float* __restrict__ logits, SampleWork w, int V, float inv_t,
-                                                           int top_k) {
+                                                           int top_k, float top_p) {
   __shared__ int tot[NCUT];
-  __shared__ unsigned long long z;
+  __shared__ unsigned long long z[1 + NMC];
   const int b = blockIdx.y, c = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const bool need_k = top_k > 0 && top_k < V;
-  const int cut = choose_cut(w, b, need_k, top_k, tot, &z);
+  const int cut = choose_cut(w, b, need_k, top_k, top_p, tot, z);
   if (cut < 0) return;
   const float* row = logits + (size_t)b * V;
   const int lo = c * w.tiles_per_chunk * TILE, hi = min(V, lo + w.tiles_per_chunk * TILE);
@@ -294,17 +320,32 @@ __global__ __launch_bounds__(SB) void chunk_collect_kernel(const float* __restri
   float dcut = kCut[0];
 #pragma unroll
   for (int j = 0; j < NCUT; ++j) if (j == cut) dcut = kCut[j];
-  uint32_t* list = w.cand + (size_t)b * CAP;
+  // Where this chunk's candidates go in the row's list: after those of the chunks before it, whose numbers the
+  // counting kernel left (no atomic on memory: thousands of them on one address took most of a millisecond).
+  // Within the chunk a counter in shared memory hands out the places.
+  __shared__ int before, fill;
+  if (threadIdx.x == 0) { before = 0; fill = 0; }
+  __syncthreads();
+  {
+    int mine = 0;
+    for (int cc = threadIdx.x; cc < c; cc += SB) mine += w.pcnt[((size_t)b * w.chunks + cc) * NCUT + cut];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+    if (lane == 0 && mine) atomicAdd(&before, mine);
+  }
+  __syncthreads();
+  uint32_t* list = w.cand + (size_t)b * CAPG + before;
+  const int room = CAPG - before;
   for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) {
     const bool in = ok && (m - x <= dcut);
     const unsigned long long mask = __ballot(in);
     if (mask) {
       const int leader = __ffsll((long long)mask) - 1;
       int base = 0;
-      if (lane == leader) base = atomicAdd(&w.ncand[b], __popcll(mask));
+      if (lane == leader) base = atomicAdd(&fill, __popcll(mask));
       base = __shfl(base, leader, 64);
       const int pos = base + __popcll(mask & ((1ull << lane) - 1ull));
-      if (in && pos < CAP) list[pos] = order_key(x);
+      if (in && pos < room) list[pos] = order_key(x);
     }
   });
 }
@@ -317,7 +358,7 @@ __global__ __launch_bounds__(ST) void row_threshold_kernel(const float* __restri
   __shared__ uint32_t list[CAP];
   __shared__ unsigned long long list_mass[CAP];
   __shared__ int tot[NCUT];
-  __shared__ unsigned long long z_sh;
+  __shared__ unsigned long long z_sh[1 + NMC];
   __shared__ uint32_t found[3];                           // threshold, top-k done, top-p done
   const int b = blockIdx.x;
   const float* row = logits + (size_t)b * V;
@@ -328,13 +369,70 @@ __global__ __launch_bounds__(ST) void row_threshold_kernel(const float* __restri
   uint32_t thr = 0;
   bool k_done = !need_k, p_done = !need_p;
   if (tid == 0) { found[0] = 0; found[1] = 0; found[2] = 0; }
-  const int cut = choose_cut(w, b, need_k, top_k, tot, &z_sh);
-  if (cut >= 0) {
-    const int n = min(w.ncand[b], CAP);
-    for (int j = tid; j < n; j += ST) list[j] = w.cand[(size_t)b * CAP + j];
+  const int cut = choose_cut(w, b, need_k, top_k, top_p, tot, z_sh);
+  const int n = cut >= 0 ? min(tot[cut], CAPG) : 0;
+  if (cut >= 0 && n > CAP) {
+    // a long list: the same bisections by the whole block over the list in memory
+    __shared__ unsigned long long wsum[ST / 64];
+    __shared__ uint32_t wmin[ST / 64];
+    const uint32_t* gl = w.cand + (size_t)b * CAPG;
+    unsigned long long* gm = w.cmass + (size_t)b * CAPG;
+    auto block_sum_u64 = [&](unsigned long long v) {
+      v = wave_sum_u64(v);
+      __syncthreads();
+      if (lane == 0) wsum[wave] = v;
+      __syncthreads();
+      unsigned long long t = 0;
+      for (int x = 0; x < ST / 64; ++x) t += wsum[x];
+      return t;
+    };
+    uint32_t kmin = 0xffffffffu;
+    for (int j = tid; j < n; j += ST) {
+      const uint32_t key = gl[j];
+      kmin = min(kmin, key);
+      if (need_p) gm[j] = fixed_mass(key_value(key), m);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) kmin = min(kmin, (uint32_t)__shfl_xor(kmin, o, 64));
+    if (lane == 0) wmin[wave] = kmin;
+    __syncthreads();                                      // also: the masses are written
+    for (int x = 0; x < ST / 64; ++x) kmin = min(kmin, wmin[x]);
+    uint32_t t = kmin;
+    if (need_k) {
+      uint32_t lo = kmin, hi = key_m;
+      while (lo < hi) {
+        const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
+        int c = 0;
+        for (int j = tid; j < n; j += ST) c += gl[j] >= mid;
+        if (block_count(c, ired) >= top_k) lo = mid; else hi = mid - 1;
+      }
+      t = lo;
+    }
+    k_done = true;
+    thr = need_k ? t : 0u;
+    if (need_p) {
+      unsigned long long kept = 0;
+      for (int j = tid; j < n; j += ST) if (gl[j] >= t) kept += gm[j];
+      kept = block_sum_u64(kept);
+      const unsigned long long z = need_k ? kept : z_sh[0];
+      const unsigned long long target = (unsigned long long)((double)top_p * (double)z);
+      if (kept > target) {
+        uint32_t lo = t, hi = key_m;
+        while (lo < hi) {
+          const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
+          unsigned long long sum = 0;
+          for (int j = tid; j < n; j += ST) if (gl[j] >= mid) sum += gm[j];
+          if (block_sum_u64(sum) > target) lo = mid; else hi = mid - 1;
+        }
+        thr = lo;
+        p_done = true;
+      }
+    }
+  } else if (cut >= 0) {
+    for (int j = tid; j < n; j += ST) list[j] = w.cand[(size_t)b * CAPG + j];
     __syncthreads();
     if (wave == 0) {
-      const unsigned long long z_row = z_sh;
+      const unsigned long long z_row = z_sh[0];
       uint32_t kmin = 0xffffffffu;
       for (int j = lane; j < n; j += 64) kmin = min(kmin, list[j]);
 #pragma unroll
@@ -582,8 +680,8 @@ extern "C" long alice_sample_workspace(int B, int V) {
   int chunks, tiles, per;
   sample_shape(B > 0 ? B : 1, V, &chunks, &tiles, &per);
   const long rows = B > 0 ? B : 1;
-  // pmass first (8-byte elements), then the 4-byte arrays
-  return rows * chunks * 2 + rows * chunks + rows * chunks * NCUT + rows + rows * CAP + rows + rows * tiles * 2 + 16;
+  // pmass and cmass first (8-byte elements), then the 4-byte arrays
+  return rows * chunks * 2 * (1 + NMC) + rows * CAPG * 2 + rows * chunks + rows * chunks * NCUT + rows * CAPG + rows + rows * tiles * 2 + 16;
 }
 
 extern "C" int alice_sample(const float* logits, int* out, const float* uniform, void* work, int B, int V,
@@ -598,11 +696,11 @@ extern "C" int alice_sample(const float* logits, int* out, const float* uniform,
   sample_shape(B, V, &w.chunks, &w.tiles, &w.tiles_per_chunk);
   const size_t rows = (size_t)B;
   w.pmass = (unsigned long long*)work;
-  w.pmax = (float*)(w.pmass + rows * w.chunks);
+  w.cmass = w.pmass + rows * w.chunks * (1 + NMC);
+  w.pmax = (float*)(w.cmass + rows * CAPG);
   w.pcnt = (int*)(w.pmax + rows * w.chunks);
-  w.ncand = w.pcnt + rows * w.chunks * NCUT;
-  w.cand = (uint32_t*)(w.ncand + rows);
-  w.thr = w.cand + rows * CAP;
+  w.cand = (uint32_t*)(w.pcnt + rows * w.chunks * NCUT);
+  w.thr = w.cand + rows * CAPG;
   w.tsum = (float*)(w.thr + rows);
   w.tlast = (int*)(w.tsum + rows * w.tiles);
   const float inv_t = 1.f / temperature;
@@ -614,7 +712,7 @@ extern "C" int alice_sample(const float* logits, int* out, const float* uniform,
     chunk_max_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t);                                                   \
     if (filtered) {                                                                                                         \
       chunk_count_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, need_k ? 0 : 1);                               \
-      chunk_collect_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, top_k);                                      \
+      chunk_collect_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, top_k, top_p);                                   \
       row_threshold_kernel<VEC><<<B, ST, 0, stream>>>(logits, w, V, inv_t, top_k, top_p);                                   \
     }                                                                                                                       \
     tile_sum_kernel<VEC><<<cgrid, SB, 0, stream>>>(logits, w, V, inv_t, filtered);                                          \

@@ -354,7 +354,8 @@ def test_sample_where_the_kept_set_is_large_or_tied(V):
     holes = rnd(B, V, seed=18, scale=3.0).cpu()
     holes[:, ::3] = -math.inf                                         # masked tokens are never drawn
     wide = rnd(B, V, seed=19, scale=0.5).cpu()                        # a nucleus of most of the vocabulary
-    for logits in (flat, steps, peaks, holes, wide):
+    broad = rnd(B, V, seed=23, scale=2.0).cpu()                       # a kept set of some thousands: the list in memory
+    for logits in (flat, steps, peaks, holes, wide, broad):
         logits = logits.to(DEV)
         for temperature, top_k, top_p in ((1.0, 0, 0.9), (1.0, 7, 1.0), (0.9, V - 1, 0.95), (1.3, 6000, 0.999),
                                           (1.0, 2, 0.6), (0.5, 0, 0.3)):
