@@ -431,18 +431,23 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
     for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC) * TM + j) * 64 + lane];
 #pragma unroll
     for (int kc = 0; kc < KC; ++kc) {
+      const int kt_next = kt_base + (s + 1) * KC + kc;       // what this k-tile's weight registers hold next
+      const bool kok = kt_next < kt_end;
 #pragma unroll
-      for (int j = 0; j < TM; ++j) {
+      for (int i = 0; i < WN; ++i) {
 #pragma unroll
-        for (int i = 0; i < WN; ++i) acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
-        // this token tile's fragment has had its last use: read the next k-tile's into the same registers
-        if (kc + 1 < KC) xf[j] = xs[(((s & 1) * KC + kc + 1) * TM + j) * 64 + lane];
-      }
-      if (more) {
-        // this k-tile's weight registers are free again: fetch the same slot of the next stage
-        __builtin_amdgcn_sched_barrier(0);
-        w_load((s + 1) * KC + kc, wk[kc]);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < TM; ++j) {
+          acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
+          // this token tile's fragment has had its last use: read the next k-tile's into the same registers
+          if (i == WN - 1 && kc + 1 < KC) xf[j] = xs[(((s & 1) * KC + kc + 1) * TM + j) * 64 + lane];
+        }
+        if (more) {
+          // this weight tile's registers are free again: fetch the same tile of the next stage now, so that the
+          // loads of a stage are spread over its products instead of arriving at the memory system in a burst
+          __builtin_amdgcn_sched_barrier(0);
+          wk[kc][i] = *reinterpret_cast<const u32x4*>(kok ? wsrc[i] + (size_t)kt_next * 512 : zero);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
   };
