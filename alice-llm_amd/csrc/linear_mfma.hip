@@ -128,7 +128,18 @@ __device__ __forceinline__ RopeToken rope_token(const RopeArgs& ra, int m) {
 // features are two whole rotated pairs (or four elements of a value head).  The sums are rounded to bfloat16
 // before the rotation, as they are when the projection and the rotation are separate kernels: both ways give
 // the same bits.
-__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc) {
+// The cosines and sines of the two pairs that features n .. n+3 make (nothing for a value head).
+struct RopeTrig { float2 c, s; };
+__device__ __forceinline__ RopeTrig rope_trig(const RopeArgs& ra, const RopeToken& t, int n) {
+  RopeTrig g{float2{1.f, 1.f}, float2{0.f, 0.f}};
+  const int d = ra.d, head = n / d, p0 = (n % d) >> 1;
+  if (head < ra.nH + ra.nKV) {
+    g.c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)t.pos * (d >> 1) + p0);
+    g.s = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)t.pos * (d >> 1) + p0);
+  }
+  return g;
+}
+__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc, const RopeTrig& tr) {
   const int d = ra.d, half = d >> 1;
   const int head = n / d, w = n % d;
   float x[4];
@@ -136,11 +147,9 @@ __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const Rop
   for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[e]);
   if (head < ra.nH + ra.nKV) {
     const int p0 = w >> 1;                                 // the pairs p0 and p0 + 1 of the head
-    const float2 c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)t.pos * half + p0);
-    const float2 sn = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)t.pos * half + p0);
     float l0, h0, l1, h1;
-    rotate_pair(x[0], x[1], c.x, sn.x, l0, h0);
-    rotate_pair(x[2], x[3], c.y, sn.y, l1, h1);
+    rotate_pair(x[0], x[1], tr.c.x, tr.s.x, l0, h0);
+    rotate_pair(x[2], x[3], tr.c.y, tr.s.y, l1, h1);
     const uint32_t lo = pack_bf16x2(l0, l1), hi = pack_bf16x2(h0, h1);
     if (head < ra.nH) {
       bf16_t* dst = ra.q_out + ((size_t)m * ra.nH + head) * d;
@@ -156,6 +165,9 @@ __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const Rop
 #pragma unroll
     for (int e = 0; e < 4; ++e) dst[v_offset(ra.layout, t.tp, w + e, d)] = f32_to_bf16(x[e]);
   }
+}
+__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc) {
+  rope_store4(ra, m, t, n, acc, rope_trig(ra, t, n));
 }
 
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
@@ -464,14 +476,25 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
   }
 
   if constexpr (EPI == ALICE_EPI_ROPE) {
+    // Every token's place first, then the cosines and sines one token tile ahead of the stores: the loads of a
+    // tile are independent and in flight together, instead of a chain of round trips between the stores.
+    RopeToken tk[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) tk[j] = rope_token(ra, min(m0 + j * 16 + r, M - 1));
+    RopeTrig tr[2][WN];
+    auto trig = [&](int j, RopeTrig (&o)[WN]) {
+#pragma unroll
+      for (int i = 0; i < WN; ++i) o[i] = rope_trig(ra, tk[j], min(tile[i], NT - 1) * 16 + g * 4);
+    };
+    trig(0, tr[0]);
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
+      if (j + 1 < TM) trig(j + 1, tr[(j + 1) & 1]);
       const int m = m0 + j * 16 + r;
       if (m >= M) continue;
-      const RopeToken t = rope_token(ra, m);
 #pragma unroll
       for (int i = 0; i < WN; ++i)
-        if (tile[i] < NT) rope_store4(ra, m, t, tile[i] * 16 + g * 4, acc[i][j]);
+        if (tile[i] < NT) rope_store4(ra, m, tk[j], tile[i] * 16 + g * 4, acc[i][j], tr[j & 1][i]);
     }
     return;
   }
