@@ -97,7 +97,7 @@ __device__ __forceinline__ float block_inclusive_scan(float v, float* wred, floa
 //   chunk_max        the maximum of every chunk
 //   chunk_count      how many elements of the chunk lie within fixed distances of the row's maximum (and, for
 //                    top-p alone, the chunk's probability mass)
-//   chunk_collect    the elements within the chosen distance (at most CAPG a row) go to the row's list
+//   chunk_collect    the elements within the chosen distance (at most capg a row) go to the row's list
 //   row_threshold    the thresholds of top-k and top-p by bisection on the key space over that list, held in
 //                    shared memory (up to CAP candidates: one wave does it) or read from memory by the whole
 //                    block; probabilities enter as 64-bit fixed point, so the sums do not depend on the
@@ -110,7 +110,7 @@ __device__ __forceinline__ float block_inclusive_scan(float v, float* wred, floa
 // thread per load where the vocabulary is a multiple of four.
 constexpr int TILE = 4096;       // 4 consecutive elements per thread of the draw's scan
 constexpr int CAP = 4096;        // candidates held in shared memory
-constexpr int CAPG = 32768;      // candidates of a row's list in memory
+constexpr int CAPG = 32768;      // candidates of a row's list in memory, at most (fewer for very many rows: list_room())
 constexpr int NCUT = 12;
 constexpr int SB = 256;          // threads of the per-chunk kernels
 constexpr int NMC = 4;           // distances at which the mass inside is summed too (top-p alone)
@@ -143,12 +143,12 @@ struct SampleWork {
   float* pmax;                   // [B][chunks]
   int* pcnt;                     // [B][chunks][NCUT]
   unsigned long long* pmass;     // [B][chunks][1 + NMC]: the chunk's mass, and its mass within kCut[kMassCut[i]] of the maximum
-  uint32_t* cand;                // [B][CAPG]
-  unsigned long long* cmass;     // [B][CAPG]: the candidates' masses, for lists too long for shared memory
+  uint32_t* cand;                // [B][capg]
+  unsigned long long* cmass;     // [B][capg]: the candidates' masses, for lists too long for shared memory
   uint32_t* thr;                 // [B]
   float* tsum;                   // [B][tiles]
   int* tlast;                    // [B][tiles]
-  int chunks, tiles, tiles_per_chunk;
+  int chunks, tiles, tiles_per_chunk, capg;
 };
 
 // f(index, logit / T, valid) for the elements [lo, hi) of a row (lo a multiple of four); every lane of the block
@@ -291,15 +291,15 @@ __device__ __forceinline__ int choose_cut(const SampleWork& w, int b, bool need_
 #pragma unroll
     for (int i = 0; i < NMC; ++i) {
       const int c = tot[kMassCut[i]];
-      if (cut == -1 && c >= 1 && c <= CAPG && z[1 + i] > target + (target >> 16)) cut = kMassCut[i];
+      if (cut == -1 && c >= 1 && c <= w.capg && z[1 + i] > target + (target >> 16)) cut = kMassCut[i];
     }
     if (cut >= 0) return cut;
   }
 #pragma unroll
   for (int j = 0; j < NCUT; ++j) {
     const int c = tot[j];
-    if (need_k) { if (cut == -1 && c >= top_k && c <= CAPG) cut = j; if (cut == -1 && c > CAPG) cut = -2; }
-    else if (c >= 1 && c <= CAPG) cut = j;
+    if (need_k) { if (cut == -1 && c >= top_k && c <= w.capg) cut = j; if (cut == -1 && c > w.capg) cut = -2; }
+    else if (c >= 1 && c <= w.capg) cut = j;
   }
   return cut;
 }
@@ -334,8 +334,8 @@ __global__ __launch_bounds__(SB) void chunk_collect_kernel(const float* __restri
     if (lane == 0 && mine) atomicAdd(&before, mine);
   }
   __syncthreads();
-  uint32_t* list = w.cand + (size_t)b * CAPG + before;
-  const int room = CAPG - before;
+  uint32_t* list = w.cand + (size_t)b * w.capg + before;
+  const int room = w.capg - before;
   for_range<VEC, SB>(row, lo, hi, inv_t, [&](int, float x, bool ok) {
     const bool in = ok && (m - x <= dcut);
     const unsigned long long mask = __ballot(in);
@@ -370,13 +370,13 @@ __global__ __launch_bounds__(ST) void row_threshold_kernel(const float* __restri
   bool k_done = !need_k, p_done = !need_p;
   if (tid == 0) { found[0] = 0; found[1] = 0; found[2] = 0; }
   const int cut = choose_cut(w, b, need_k, top_k, top_p, tot, z_sh);
-  const int n = cut >= 0 ? min(tot[cut], CAPG) : 0;
+  const int n = cut >= 0 ? min(tot[cut], w.capg) : 0;
   if (cut >= 0 && n > CAP) {
     // a long list: the same bisections by the whole block over the list in memory
     __shared__ unsigned long long wsum[ST / 64];
     __shared__ uint32_t wmin[ST / 64];
-    const uint32_t* gl = w.cand + (size_t)b * CAPG;
-    unsigned long long* gm = w.cmass + (size_t)b * CAPG;
+    const uint32_t* gl = w.cand + (size_t)b * w.capg;
+    unsigned long long* gm = w.cmass + (size_t)b * w.capg;
     auto block_sum_u64 = [&](unsigned long long v) {
       v = wave_sum_u64(v);
       __syncthreads();
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(ST) void row_threshold_kernel(const float* __restri
       }
     }
   } else if (cut >= 0) {
-    for (int j = tid; j < n; j += ST) list[j] = w.cand[(size_t)b * CAPG + j];
+    for (int j = tid; j < n; j += ST) list[j] = w.cand[(size_t)b * w.capg + j];
     __syncthreads();
     if (wave == 0) {
       const unsigned long long z_row = z_sh[0];
@@ -640,6 +640,13 @@ __global__ __launch_bounds__(ST) void draw_kernel(const float* __restrict__ logi
   if (tid == 0) out[b] = pick[0] >= 0 ? pick[0] : max(pick[1], 0);
 }
 
+// How long a row's list may be: 32,768 candidates, fewer (down to what fits shared memory) when the lists of
+// all rows would take more than 200 MB.
+__host__ inline int list_room(int B) {
+  long room = (16L << 20) / (B > 0 ? B : 1);
+  return (int)(room > CAPG ? CAPG : (room < CAP ? CAP : room));
+}
+
 // chunks, tiles and tiles per chunk of a call
 __host__ inline void sample_shape(int B, int V, int* chunks, int* tiles, int* per) {
   *tiles = (V + TILE - 1) / TILE;
@@ -681,7 +688,8 @@ extern "C" long alice_sample_workspace(int B, int V) {
   sample_shape(B > 0 ? B : 1, V, &chunks, &tiles, &per);
   const long rows = B > 0 ? B : 1;
   // pmass and cmass first (8-byte elements), then the 4-byte arrays
-  return rows * chunks * 2 * (1 + NMC) + rows * CAPG * 2 + rows * chunks + rows * chunks * NCUT + rows * CAPG + rows + rows * tiles * 2 + 16;
+  const long capg = list_room(B);
+  return rows * chunks * 2 * (1 + NMC) + rows * capg * 2 + rows * chunks + rows * chunks * NCUT + rows * capg + rows + rows * tiles * 2 + 16;
 }
 
 extern "C" int alice_sample(const float* logits, int* out, const float* uniform, void* work, int B, int V,
@@ -694,13 +702,14 @@ extern "C" int alice_sample(const float* logits, int* out, const float* uniform,
   if (B == 0) return 0;
   SampleWork w;
   sample_shape(B, V, &w.chunks, &w.tiles, &w.tiles_per_chunk);
+  w.capg = list_room(B);
   const size_t rows = (size_t)B;
   w.pmass = (unsigned long long*)work;
   w.cmass = w.pmass + rows * w.chunks * (1 + NMC);
-  w.pmax = (float*)(w.cmass + rows * CAPG);
+  w.pmax = (float*)(w.cmass + rows * w.capg);
   w.pcnt = (int*)(w.pmax + rows * w.chunks);
   w.cand = (uint32_t*)(w.pcnt + rows * w.chunks * NCUT);
-  w.thr = w.cand + rows * CAPG;
+  w.thr = w.cand + rows * w.capg;
   w.tsum = (float*)(w.thr + rows);
   w.tlast = (int*)(w.tsum + rows * w.tiles);
   const float inv_t = 1.f / temperature;
