@@ -128,20 +128,25 @@ __device__ __forceinline__ RopeToken rope_token(const RopeArgs& ra, int m) {
 // features are two whole rotated pairs (or four elements of a value head).  The sums are rounded to bfloat16
 // before the rotation, as they are when the projection and the rotation are separate kernels: both ways give
 // the same bits.
-// The cosines and sines of the two pairs that features n .. n+3 make (nothing for a value head).
+// Which head features n .. n+3 belong to and where in it they lie: the same for every token of a tile, so the
+// divisions by the head size are done once per tile, not per token.
+struct RopeCol { int head, w; };
+__device__ __forceinline__ RopeCol rope_col(const RopeArgs& ra, int n) { return RopeCol{n / ra.d, n % ra.d}; }
+
+// The cosines and sines of the two pairs that the four features make (nothing for a value head).
 struct RopeTrig { float2 c, s; };
-__device__ __forceinline__ RopeTrig rope_trig(const RopeArgs& ra, const RopeToken& t, int n) {
+__device__ __forceinline__ RopeTrig rope_trig(const RopeArgs& ra, const RopeToken& t, const RopeCol& col) {
   RopeTrig g{float2{1.f, 1.f}, float2{0.f, 0.f}};
-  const int d = ra.d, head = n / d, p0 = (n % d) >> 1;
-  if (head < ra.nH + ra.nKV) {
-    g.c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)t.pos * (d >> 1) + p0);
-    g.s = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)t.pos * (d >> 1) + p0);
+  if (col.head < ra.nH + ra.nKV) {
+    g.c = *reinterpret_cast<const float2*>(ra.cos_t + (size_t)t.pos * (ra.d >> 1) + (col.w >> 1));
+    g.s = *reinterpret_cast<const float2*>(ra.sin_t + (size_t)t.pos * (ra.d >> 1) + (col.w >> 1));
   }
   return g;
 }
-__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc, const RopeTrig& tr) {
+__device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, const RopeCol& col, f32x4 acc,
+                                            const RopeTrig& tr) {
   const int d = ra.d, half = d >> 1;
-  const int head = n / d, w = n % d;
+  const int head = col.head, w = col.w;
   float x[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[e]);
@@ -167,7 +172,8 @@ __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const Rop
   }
 }
 __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const RopeToken& t, int n, f32x4 acc) {
-  rope_store4(ra, m, t, n, acc, rope_trig(ra, t, n));
+  const RopeCol col = rope_col(ra, n);
+  rope_store4(ra, m, t, col, acc, rope_trig(ra, t, col));
 }
 
 // ---------------------------------------------------------------- weight streaming, M <= 16*MT
@@ -481,10 +487,13 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
     RopeToken tk[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) tk[j] = rope_token(ra, min(m0 + j * 16 + r, M - 1));
+    RopeCol col[WN];
+#pragma unroll
+    for (int i = 0; i < WN; ++i) col[i] = rope_col(ra, min(tile[i], NT - 1) * 16 + g * 4);
     RopeTrig tr[2][WN];
     auto trig = [&](int j, RopeTrig (&o)[WN]) {
 #pragma unroll
-      for (int i = 0; i < WN; ++i) o[i] = rope_trig(ra, tk[j], min(tile[i], NT - 1) * 16 + g * 4);
+      for (int i = 0; i < WN; ++i) o[i] = rope_trig(ra, tk[j], col[i]);
     };
     trig(0, tr[0]);
 #pragma unroll
@@ -494,7 +503,7 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
       if (m >= M) continue;
 #pragma unroll
       for (int i = 0; i < WN; ++i)
-        if (tile[i] < NT) rope_store4(ra, m, tk[j], tile[i] * 16 + g * 4, acc[i][j], tr[j & 1][i]);
+        if (tile[i] < NT) rope_store4(ra, m, tk[j], col[i], acc[i][j], tr[j & 1][i]);
     }
     return;
   }
