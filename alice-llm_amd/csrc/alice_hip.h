@@ -33,6 +33,8 @@ extern "C" {
 
 const char* alice_last_error();
 int alice_abi_version();
+// Digest of the sources and flags this library was built from; the bindings compare it with the sources beside them.
+const char* alice_source_digest();
 int alice_device_arch(char* out, int cap);
 
 int alice_embed(const int* tokens, const void* table, int table_dtype, int table_layout, float* out,

@@ -4,6 +4,7 @@ built, and by the repository's build entry point, which compiles every time."""
 from __future__ import annotations
 
 import concurrent.futures as cf
+import hashlib
 import os
 import shutil
 import subprocess
@@ -21,6 +22,17 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-ta
 
 def sources():
     return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
+
+
+def source_digest() -> str:
+    """A digest of everything the library is made from (sources, headers, compiler flags).  It is compiled
+    into the library, so that a library built from other sources than the ones beside it is noticed."""
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    for f in sorted(f for f in os.listdir(HERE) if f.endswith((".hip", ".h"))):
+        h.update(f.encode())
+        with open(os.path.join(HERE, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:32]
 
 
 def _hipcc() -> str:
@@ -45,25 +57,27 @@ def _writable(path: str) -> bool:
 def output_dirs():
     """Where the library is looked for and built: in the tree first, else a per-user temp folder."""
     in_tree = os.path.join(os.path.dirname(HERE), "hip")
-    fallback = os.path.join(tempfile.gettempdir(), f"alice_llm_amd_{os.getuid()}")
+    fallback = os.path.join(tempfile.gettempdir(), f"alice_llm_amd_{os.getuid()}", source_digest())
     return [in_tree, fallback]
 
 
+def built_libraries():
+    """Every built library there is, in the order of preference."""
+    return [p for p in (os.path.join(d, LIB_NAME) for d in output_dirs()) if os.path.exists(p)]
+
+
 def find_library():
-    for d in output_dirs():
-        p = os.path.join(d, LIB_NAME)
-        if os.path.exists(p):
-            return p
-    return None
+    libs = built_libraries()
+    return libs[0] if libs else None
 
 
 def _say(msg: str) -> None:
     print(f"[alice-llm_amd build] {msg}", file=sys.stderr, flush=True)
 
 
-def _compile(hipcc: str, src: str, obj: str) -> float:
+def _compile(hipcc: str, src: str, obj: str, digest: str) -> float:
     t0 = time.time()
-    cmd = [hipcc, *FLAGS, "-c", os.path.join(HERE, src), "-o", obj]
+    cmd = [hipcc, *FLAGS, f'-DALICE_SOURCE_DIGEST="{digest}"', "-c", os.path.join(HERE, src), "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr[-4000:]}")
@@ -79,6 +93,7 @@ def build(verbose: bool = True) -> str:
     obj_dir = os.path.join(out_dir, "_build")
     os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
+    digest = source_digest()
     if verbose:
         _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
     # object files carry the process id: two processes that build at once (a test runner and a program it
@@ -87,7 +102,7 @@ def build(verbose: bool = True) -> str:
     t0 = time.time()
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or (os.cpu_count() or 4), 16))
     with cf.ThreadPoolExecutor(workers) as pool:
-        futs = {pool.submit(_compile, hipcc, s, o): s for s, o in objs.items()}
+        futs = {pool.submit(_compile, hipcc, s, o, digest): s for s, o in objs.items()}
         pending = set(futs)
         while pending:
             done, pending = cf.wait(pending, timeout=15, return_when=cf.FIRST_COMPLETED)

@@ -17,6 +17,12 @@ extern "C" const char* alice_last_error() { return g_error; }
 
 extern "C" int alice_abi_version() { return ALICE_ABI_VERSION; }
 
+// The digest of the sources that this library was built from (given by the build script).
+#ifndef ALICE_SOURCE_DIGEST
+#define ALICE_SOURCE_DIGEST ""
+#endif
+extern "C" const char* alice_source_digest() { return ALICE_SOURCE_DIGEST; }
+
 // The architecture name of the current device, e.g. "gfx950:sramecc+:xnack-".
 extern "C" int alice_device_arch(char* out, int cap) {
   int dev = 0;

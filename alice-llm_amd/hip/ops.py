@@ -21,6 +21,7 @@ LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED256 = 0, 1,
 ABI_VERSION = 4
 
 _lib = None
+_lib_path = None
 _lock = threading.Lock()
 
 
@@ -59,29 +60,51 @@ def _declare(lib) -> None:
         fn.restype = I
 
 
+def _open(path: str):
+    try:
+        return ctypes.CDLL(path)
+    except OSError as e:
+        raise HipLibraryError(f"cannot load {path}: {e}") from e
+
+
+def _built_from_these_sources(lib) -> bool:
+    try:
+        fn = lib.alice_source_digest
+    except AttributeError:
+        return False
+    fn.restype = ctypes.c_char_p
+    return fn().decode() == _build.source_digest()
+
+
 def library():
-    """The loaded HIP library; built with hipcc at the first call if no built one is found."""
-    global _lib
+    """The loaded HIP library: the built one if it was made from the sources beside these bindings, else
+    built with hipcc at the first call."""
+    global _lib, _lib_path
     if _lib is not None:
         return _lib
     with _lock:
         if _lib is not None:
             return _lib
-        path = _build.find_library()
-        if path is None:
+        lib = path = None
+        for cand in _build.built_libraries():
+            found = _open(cand)
+            if _built_from_these_sources(found):
+                lib, path = found, cand
+                break
+            # a library left from other sources (an older checkout's, an edit after the last build) would give
+            # results that belong to no version of the code: it is never used
+            _build._say(f"{cand} was built from other sources than the ones beside it")
+        if lib is None:
             try:
                 path = _build.build(verbose=True)
             except Exception as e:
                 raise HipLibraryError(f"the HIP library is not built and building it failed: {e}") from e
-        try:
-            lib = ctypes.CDLL(path)
-        except OSError as e:
-            raise HipLibraryError(f"cannot load {path}: {e}") from e
+            lib = _open(path)
         _declare(lib)
         if lib.alice_abi_version() != ABI_VERSION:
             raise HipLibraryError(f"{path} has interface version {lib.alice_abi_version()}, these bindings "
                                   f"need {ABI_VERSION}: rebuild it (python -m alice_llm_amd.csrc.build)")
-        _lib = lib
+        _lib, _lib_path = lib, path
         return _lib
 
 
@@ -92,7 +115,8 @@ def library_ready() -> bool:
 
 
 def library_path() -> Optional[str]:
-    return _build.find_library()
+    """The library in use, or the one that would be tried first."""
+    return _lib_path or _build.find_library()
 
 
 def require_gpu() -> torch.device:

@@ -151,3 +151,32 @@ def test_sharded_folder(tmp_path):
     (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"x.weight": "missing.safetensors"}}))
     with pytest.raises(WeightFileError, match="missing.safetensors"):
         TensorSource(str(tmp_path))
+
+
+def test_a_library_from_other_sources_is_not_used(tmp_path, monkeypatch):
+    """The library carries a digest of its sources and flags: the bindings use a built library only if the
+    digest is that of the sources beside them (a library left from an edit or an older checkout is not)."""
+    from alice_llm_amd.csrc import build
+    from alice_llm_amd.hip import ops
+    d0 = build.source_digest()
+    assert len(d0) == 32 and d0 == build.source_digest()
+    src = tmp_path / "csrc"
+    src.mkdir()
+    (src / "a.hip").write_text("int x;")
+    (src / "a.h").write_text("")
+    monkeypatch.setattr(build, "HERE", str(src))
+    d1 = build.source_digest()
+    (src / "a.h").write_text("// edited")
+    d2 = build.source_digest()
+    monkeypatch.setattr(build, "FLAGS", build.FLAGS + ["-O0"])
+    assert len({d0, d1, d2, build.source_digest()}) == 4
+
+    class Old:                                    # a library from before the digest existed
+        pass
+
+    class Built:
+        def __init__(self, d):
+            self.alice_source_digest = lambda: d.encode()
+    assert not ops._built_from_these_sources(Old())
+    assert not ops._built_from_these_sources(Built(d2))
+    assert ops._built_from_these_sources(Built(build.source_digest()))
