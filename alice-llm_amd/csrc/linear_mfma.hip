@@ -560,8 +560,8 @@ __device__ __forceinline__ void wait_vmcnt() {               // s_waitcnt vmcnt(
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int EPI, typename TO, bool FULL, bool XF>
-__global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
+template <int EPI, typename TO, bool FULL, bool XF, int FI>
+__global__ __launch_bounds__(128 * (8 / FI), 1) void linear_tiled256_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                                  TO* __restrict__ y, int M, int N, int K, int KT, int NT,
                                                                  float epi, int gx, int gy, int kt_per_slice, int y_frag,
                                                                  RopeArgs ra) {
@@ -570,7 +570,8 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int r32 = lane & 31, h = lane >> 5, upper = (lane >> 4) & 1;
-  const int wm = wave & 1, wn = wave >> 1;                   // this wave's half of the tokens and of the features
+  constexpr int NW = 2 * (8 / FI), TPW = 32 / NW;            // waves; tiles of a k-tile that a wave brings
+  const int wm = wave & 1, wn = wave >> 1;                   // this wave's half of the tokens, its share of the features
   const int id = blockIdx.x, xcd = id & 7, local = id >> 3;  // XCD x works through the x-th eighth of the blocks
   const int per = (gx * gy + 7) >> 3;
   const int item = xcd * per + local;
@@ -586,27 +587,29 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
     }
     return (bx * 2 + hf) * 8 + i;
   };
-  int tile[8];
+  int tile[2 * FI];                                          // the 16-row weight tiles of this wave's features
 #pragma unroll
-  for (int i = 0; i < 8; ++i) tile[i] = tile_of(wn, i);
-  // What this wave brings per k-tile: waves 0 and 1 the token tiles 8 wave .. + 7, waves 2 and 3 the weight tiles
-  // of feature half wave - 2.  One address per tile and lane at k-tile 0; all loads are unconditional (rows and
-  // tiles beyond the matrix are clamped, k-tiles beyond the slice bring the zero tile or the last k-tile again).
-  const bool brings_x = wave < 2;
-  const bf16_t* src[8];
+  for (int i = 0; i < 2 * FI; ++i) tile[i] = tile_of((2 * FI * wn + i) >> 3, (2 * FI * wn + i) & 7);
+  // What this wave brings per k-tile: the ring's tiles TPW wave .. + TPW - 1, of which the first 16 are token tiles
+  // and the other 16 the weight tiles of the two feature halves.  One address per tile and lane at k-tile 0; all
+  // loads are unconditional (rows and tiles beyond the matrix are clamped, k-tiles beyond the slice bring the zero
+  // tile or the last k-tile again).
+  const int slot_base = TPW * wave;
+  const bool brings_x = slot_base < 16;
+  const bf16_t* src[TPW];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < TPW; ++i) {
+    const int xt = (slot_base + i) & 15, wt = (slot_base + i) & 15;
     const bf16_t* xs;
-    if constexpr (XF) xs = x + ((size_t)min((m0 >> 4) + 8 * (wave & 1) + i, (M - 1) >> 4) * KT * 64 + lane) * 8;
-    else xs = x + (size_t)min(m0 + (8 * (wave & 1) + i) * 16 + r, M - 1) * K;
-    const bf16_t* ws = wf + (size_t)min(tile_of(wave & 1, i), NT - 1) * KT * 512 + lane * 8;
+    if constexpr (XF) xs = x + ((size_t)min((m0 >> 4) + xt, (M - 1) >> 4) * KT * 64 + lane) * 8;
+    else xs = x + (size_t)min(m0 + xt * 16 + r, M - 1) * K;
+    const bf16_t* ws = wf + (size_t)min(tile_of(wt >> 3, wt & 7), NT - 1) * KT * 512 + lane * 8;
     src[i] = brings_x ? xs : ws;
   }
   const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
   const int kt_base = blockIdx.y * kt_per_slice, kt_end = min(KT, kt_base + kt_per_slice);
   const int T = kt_end - kt_base;
   y += (size_t)blockIdx.y * M * N;
-  const int slot_base = brings_x ? 8 * wave : 16 + 8 * (wave - 2);
   auto bring = [&](int rel) {                                // k-tile kt_base + rel into ring slot rel % RING
     const int kt = kt_base + rel;
     const bool kok = kt < kt_end;
@@ -616,16 +619,16 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
     else off = (size_t)ktc * 512;
     u32x4* dst = ring + ((size_t)(rel % RING) * 32 + slot_base) * 64;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TPW; ++i) {
       const bf16_t* p = (brings_x || kok) ? src[i] + off : zero;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
                                        (__attribute__((address_space(3))) void*)(dst + i * 64), 16, 0, 0);
     }
   };
 
-  f32x16 acc[4][4];                                          // [feature tile of 32][token tile of 32]
+  f32x16 acc[FI][4];                                         // [feature tile of 32][token tile of 32]
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < FI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -635,47 +638,47 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
   // are read from LDS into the other and the loads of k-tile t + 3 are issued, all between the MFMAs (the
   // scheduling groups below fix that order; left alone, the compiler puts the reads in front and the wave,
   // the only one of its SIMD, waits for them).  A k-tile beyond the slice brings zero weights and adds nothing.
-  u32x4 xa[2][4], wa[2][4], xb[2][4], wb[2][4];
+  u32x4 xa[2][4], wa[2][FI], xb[2][4], wb[2][FI];
   const int piece = h * 16 + r;                              // of k-half 0; k-half 1 is 32 pieces on
-  auto frags = [&](int t, u32x4 (&xf)[2][4], u32x4 (&wk)[2][4]) {
+  auto frags = [&](int t, u32x4 (&xf)[2][4], u32x4 (&wk)[2][FI]) {
     const u32x4* st = ring + (size_t)(t % RING) * 32 * 64;
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) xf[kh][j] = st[(8 * wm + 2 * j + upper) * 64 + kh * 32 + piece];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) wk[kh][i] = st[(16 + 8 * wn + 2 * i + upper) * 64 + kh * 32 + piece];
+      for (int i = 0; i < FI; ++i) wk[kh][i] = st[(16 + 2 * FI * wn + 2 * i + upper) * 64 + kh * 32 + piece];
     }
   };
-  auto products = [&](const u32x4 (&xf)[2][4], const u32x4 (&wk)[2][4]) {
+  auto products = [&](const u32x4 (&xf)[2][4], const u32x4 (&wk)[2][FI]) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i][j] = mfma32(wk[kh][i], xf[kh][j], acc[i][j]);
+        for (int i = 0; i < FI; ++i) acc[i][j] = mfma32(wk[kh][i], xf[kh][j], acc[i][j]);
   };
-  auto interleave = [&]() {                                  // 32 MFMAs, 16 LDS reads, 8 loads
+  auto interleave = [&]() {                                  // 8 FI MFMAs, 8 + 2 FI LDS reads, TPW loads
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < TPW; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, FI == 4 ? 1 : 2, 0);
     }
   };
   // A barrier instruction alone: __syncthreads() carries a fence, for which the compiler waits until every
   // load in flight has written LDS, the ones for the k-tiles ahead included.
   auto landed = [&]() {
-    wait_vmcnt<(RING - 2) * 8>();                            // all but the newest RING - 2 k-tiles asked for: this wave's part is there
+    wait_vmcnt<(RING - 2) * TPW>();                            // all but the newest RING - 2 k-tiles asked for: this wave's part is there
     asm volatile("s_barrier" ::: "memory");                  // everyone's is, and everyone is done with the k-tile before
   };
   // During the products of k-tile t (fragments in registers) the ring holds k-tile t + 1, which is being read,
   // and the RING - 1 after it, which are on their way: k-tile t + RING goes where k-tile t was.
 #pragma unroll
   for (int s = 0; s < RING; ++s) bring(s);
-  wait_vmcnt<(RING - 1) * 8>();
+  wait_vmcnt<(RING - 1) * TPW>();
   asm volatile("s_barrier" ::: "memory");
   frags(0, xa, wa);
   for (int t = 0; t < T; t += 2) {
@@ -704,7 +707,7 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
     if constexpr (EPI == ALICE_EPI_ROPE) {
       const RopeToken tk = rope_token(ra, m);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < FI; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int t16 = tile[2 * i + (q >> 1)];
@@ -714,7 +717,7 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
         }
     } else if constexpr (EPI == ALICE_EPI_GEGLU) {
 #pragma unroll
-      for (int p = 0; p < 2; ++p)
+      for (int p = 0; p < FI / 2; ++p)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int t16 = tile[4 * p + (q >> 1)];            // the gate's tile; the up half's has the same place in N
@@ -726,7 +729,7 @@ __global__ __launch_bounds__(256, 1) void linear_tiled256_kernel(const bf16_t* _
         }
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < FI; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int t16 = tile[2 * i + (q >> 1)];
@@ -820,29 +823,26 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int per = ceil_div(KT, split);
   {
-    // big: 1 forces the 256 x 256 blocks, -1 forbids them
+    // big: 1 forces the 256 x 256 blocks with four waves, 2 with eight, -1 forbids them
     const int gx256 = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 8) : ceil_div(NT, 16);
     if (big > 0 || (big == 0 && big_tiles_pay(M, gx256, split))) {
       const int gy256 = ceil_div(M, 256);
       dim3 grid(8 * ceil_div(gx256 * gy256, 8), split);
-      static bool prepared[2] = {false, false};
-      if (x_frag) {
-        auto kern = linear_tiled256_kernel<EPI, TO, false, true>;
-        if (!prepared[1]) {
-          ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) == hipSuccess,
-                      "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
-          prepared[1] = true;
+      auto go = [&](auto kern, int threads, bool& prepared) {
+        if (!prepared) {
+          if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) != hipSuccess) return false;
+          prepared = true;
         }
-        kern<<<grid, 256, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
-      } else {
-        auto kern = linear_tiled256_kernel<EPI, TO, false, false>;
-        if (!prepared[0]) {
-          ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) == hipSuccess,
-                      "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
-          prepared[0] = true;
-        }
-        kern<<<grid, 256, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
-      }
+        kern<<<grid, threads, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
+        return true;
+      };
+      static bool prepared[4] = {false, false, false, false};
+      bool ok;
+      if (big == 2) ok = x_frag ? go(linear_tiled256_kernel<EPI, TO, false, true, 2>, 512, prepared[3])
+                                : go(linear_tiled256_kernel<EPI, TO, false, false, 2>, 512, prepared[2]);
+      else ok = x_frag ? go(linear_tiled256_kernel<EPI, TO, false, true, 4>, 256, prepared[1])
+                       : go(linear_tiled256_kernel<EPI, TO, false, false, 4>, 256, prepared[0]);
+      ALICE_CHECK(ok, "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
       ALICE_LAUNCH_CHECK();
       return 0;
     }
@@ -948,7 +948,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
     }                                                                                              \
   } while (0)
   if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
-  const int big = variant == ALICE_LINEAR_TILED256 ? 1 : (variant == ALICE_LINEAR_MFMA ? -1 : 0);
+  const int big = variant == ALICE_LINEAR_TILED256 ? 1 : variant == ALICE_LINEAR_TILED256W8 ? 2 : (variant == ALICE_LINEAR_MFMA ? -1 : 0);
   BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream, RopeArgs{}, big);
 #undef BY_EPI
 }
