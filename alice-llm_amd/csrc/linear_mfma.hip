@@ -108,6 +108,16 @@ struct RopeArgs {
   int bt_stride, nH, nKV, d, page_size, n_pages, layout;
 };
 
+// A token as the tiled kernel's rotation epilogue keeps it in LDS, and the elements per staged token there: 256
+// features and 8 of padding (a token's stride is 132 words, so that neither 64 lanes on 16 tokens x 4 words nor 16
+// tokens x 16 bytes meet in a bank).
+struct RopeStagedToken {
+  size_t page_base;
+  int tp;
+  bool valid, page_ok;
+};
+constexpr int ROPE_PITCH = 264;
+
 // Where token m's keys and values go.
 struct RopeToken {
   int pos, tp;
@@ -363,7 +373,10 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
                                                                float epi, int gx, int gy, int kt_per_slice, int y_frag,
                                                                RopeArgs ra) {
   constexpr int XJ = TM / 4;                               // token tiles each wave stages
-  __shared__ __align__(16) uint32_t xs_raw[2 * KC * TM * 64 * 4];
+  // The rotation epilogue stages 64 tokens x 256 features in the same memory afterwards (ROPE_PITCH elements a token).
+  constexpr int XS_WORDS = 2 * KC * TM * 64 * 4;
+  constexpr int LDS_WORDS = (EPI == ALICE_EPI_ROPE && XS_WORDS < 64 * ROPE_PITCH / 2) ? 64 * ROPE_PITCH / 2 : XS_WORDS;
+  __shared__ __align__(16) uint32_t xs_raw[LDS_WORDS];
   u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -482,8 +495,24 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
   }
 
   if constexpr (EPI == ALICE_EPI_ROPE) {
-    // Every token's place first, then the cosines and sines one token tile ahead of the stores: the loads of a
-    // tile are independent and in flight together, instead of a chain of round trips between the stores.
+    // The rotated values go to their places through LDS, 64 tokens at a time: a lane holds two pairs of a token
+    // (4-byte pieces of 16 different rows of q or of the cache), and stores of such pieces cost several times the
+    // product's own time per byte.  Staged, a token's 16 features of a weight tile become two runs of eight
+    // neighbouring elements of a head (the low and the high halves of eight pairs; a value head's 16 elements as
+    // they are), and every thread then moves 16-byte runs: along a token for q and for row-major caches, along 16
+    // tokens for keys in fragment order (a 1 KB tile per wave when the tokens start at a multiple of 16), and for
+    // values in fragment order eight tokens of one element at a time, which is that layout's 16-byte unit (when 32
+    // tokens are consecutive places of one sequence from a multiple of 32 on; one by one otherwise).
+    __shared__ RopeStagedToken tinfo[64];
+    __shared__ int group_ok[2];
+    bf16_t* stage = reinterpret_cast<bf16_t*>(xs_raw);
+    const int tid = threadIdx.x;
+    const int n_tile0 = bx * 4 * WN;
+    const int head0 = n_tile0 * 16 / ra.d;
+    const bool key_block = ra.layout == 1 && head0 >= ra.nH && head0 < ra.nH + ra.nKV;
+    const bool value_block = ra.layout == 1 && head0 >= ra.nH + ra.nKV;
+    // Every token's place first, then the cosines and sines one token tile ahead of their use: the loads of a
+    // tile are independent and in flight together.
     RopeToken tk[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) tk[j] = rope_token(ra, min(m0 + j * 16 + r, M - 1));
@@ -496,14 +525,114 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
       for (int i = 0; i < WN; ++i) o[i] = rope_trig(ra, tk[j], col[i]);
     };
     trig(0, tr[0]);
+    auto emit = [&](int mb, int t, int c) {                  // run c (eight elements) of staged token t
+      const int nt = n_tile0 + (c >> 1);
+      const RopeStagedToken ti = tinfo[t];
+      if (nt >= NT || !ti.valid) return;
+      const int d = ra.d, head = nt * 16 / d, w0 = nt * 16 % d;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + t * ROPE_PITCH + c * 8);
+      if (head < ra.nH) {
+        const int dim0 = (w0 >> 1) + (c & 1) * (d >> 1);
+        *reinterpret_cast<u32x4*>(ra.q_out + ((size_t)(mb + t) * ra.nH + head) * d + dim0) = v;
+      } else if (!ti.page_ok) {
+        return;
+      } else if (head < ra.nH + ra.nKV) {
+        const int dim0 = (w0 >> 1) + (c & 1) * (d >> 1);
+        bf16_t* dst = ra.k_pool + ti.page_base + (size_t)(head - ra.nH) * ra.page_size * d;
+        *reinterpret_cast<u32x4*>(dst + k_offset(ra.layout, ti.tp, dim0, d)) = v;
+      } else {
+        const int dim0 = w0 + (c & 1) * 8;
+        bf16_t* dst = ra.v_pool + ti.page_base + (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
+        if (ra.layout == 0) {
+          *reinterpret_cast<u32x4*>(dst + (size_t)ti.tp * d + dim0) = v;
+        } else {
+          const bf16_t* e8 = stage + t * ROPE_PITCH + c * 8;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dst[v_offset(1, ti.tp, dim0 + e, d)] = e8[e];
+        }
+      }
+    };
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
+      const int mb = m0 + (j & ~3) * 16;                     // the first of the 64 tokens being staged
+      if ((j & 3) == 0) {
+        __syncthreads();                                     // the memory's last readers are done
+        if (tid < 64) {
+          const int m = mb + tid, mc = min(m, M - 1), first = min(mb + (tid & 32), M - 1);
+          const RopeToken t = rope_token(ra, mc);
+          tinfo[tid] = RopeStagedToken{t.page_base, t.tp, m < M, t.page_ok};
+          const int pos0 = ra.positions[first];
+          const bool in_run = m < M && t.page_ok && ra.seq_of_token[mc] == ra.seq_of_token[first] &&
+                              t.pos == pos0 + (tid & 31) && (pos0 & 31) == 0 && (ra.page_size & 31) == 0;
+          const unsigned long long run = __ballot(in_run);
+          if (tid == 0) {
+            group_ok[0] = (run & 0xffffffffull) == 0xffffffffull;
+            group_ok[1] = (run >> 32) == 0xffffffffull;
+          }
+        }
+      }
       if (j + 1 < TM) trig(j + 1, tr[(j + 1) & 1]);
-      const int m = m0 + j * 16 + r;
-      if (m >= M) continue;
+      uint32_t* row = reinterpret_cast<uint32_t*>(stage + ((j & 3) * 16 + r) * ROPE_PITCH + wave * (16 * WN));
 #pragma unroll
-      for (int i = 0; i < WN; ++i)
-        if (tile[i] < NT) rope_store4(ra, m, tk[j], col[i], acc[i][j], tr[j & 1][i]);
+      for (int i = 0; i < WN; ++i) {
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[i][j][e]);
+        if (col[i].head < ra.nH + ra.nKV) {
+          float l0, h0, l1, h1;
+          rotate_pair(x[0], x[1], tr[j & 1][i].c.x, tr[j & 1][i].s.x, l0, h0);
+          rotate_pair(x[2], x[3], tr[j & 1][i].c.y, tr[j & 1][i].s.y, l1, h1);
+          row[i * 8 + g] = pack_bf16x2(l0, l1);              // pairs 2 g and 2 g + 1 of the tile's eight: the low halves
+          row[i * 8 + 4 + g] = pack_bf16x2(h0, h1);          // and the high halves, eight elements on
+        } else {
+          row[i * 8 + 2 * g] = pack_bf16x2(x[0], x[1]);
+          row[i * 8 + 2 * g + 1] = pack_bf16x2(x[2], x[3]);
+        }
+      }
+      if ((j & 3) != 3) continue;
+      __syncthreads();
+      if (value_block) {
+        // wave items: (32 tokens, a 16-element tile of a head); a lane takes element lane % 16 of the tokens
+        // 4 (lane / 16) .. + 3 and the same 16 further on
+#pragma unroll 1
+        for (int it = 0; it < 8; ++it) {
+          const int item = it * 4 + wave, grp = item >> 4, vt = item & 15, nt = n_tile0 + vt;
+          if (nt >= NT) continue;
+          const int d = ra.d, head = nt * 16 / d, e = nt * 16 % d + (lane & 15), a = lane >> 4;
+          const bf16_t* src = stage + (grp * 32 + 4 * a) * ROPE_PITCH + vt * 16 + (lane & 15);
+          const size_t head_off = (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
+          if (group_ok[grp]) {
+            uint16_t h[8];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              h[q] = src[q * ROPE_PITCH].bits;
+              h[4 + q] = src[(16 + q) * ROPE_PITCH].bits;
+            }
+            const u32x4 v = {h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16,
+                             h[6] | (uint32_t)h[7] << 16};
+            const RopeStagedToken ti = tinfo[grp * 32];
+            *reinterpret_cast<u32x4*>(ra.v_pool + ti.page_base + head_off + v_offset(1, ti.tp + 4 * a, e, d)) = v;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+              const int t = grp * 32 + 4 * a + (q & 3) + 16 * (q >> 2);
+              const RopeStagedToken ti = tinfo[t];
+              if (ti.valid && ti.page_ok)
+                ra.v_pool[ti.page_base + head_off + v_offset(1, ti.tp, e, d)] = src[((q & 3) + 16 * (q >> 2)) * ROPE_PITCH];
+            }
+          }
+        }
+      } else if (key_block) {
+        // wave items: (16 tokens, 32 elements of one half of a head); a lane takes run lane / 16 of token lane % 16
+#pragma unroll 1
+        for (int it = 0; it < 8; ++it) {
+          const int item = it * 4 + wave;
+          emit(mb, 16 * (item >> 3) + (lane & 15), 8 * ((item >> 1) & 3) + 2 * (lane >> 4) + (item & 1));
+        }
+      } else {
+#pragma unroll 2
+        for (int k = 0; k < 8; ++k) emit(mb, (tid >> 5) + 8 * k, tid & 31);
+      }
     }
     return;
   }
@@ -850,9 +979,9 @@ int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
   // 128 tokens a block, or 64 when that leaves most of the chip without a block (measured at N = 2304 and 4096:
-  // 216 and 256 blocks of 128 tokens beat twice as many of 64, 128 blocks do not; with the rotation epilogue,
-  // whose stores are scattered, 256 blocks of 128 tokens lose against 512 of 64)
-  const bool high = gx * gy * split >= (EPI == ALICE_EPI_ROPE ? 384 : 192) || M <= 64;
+  // 216 and 256 blocks of 128 tokens beat twice as many of 64, 128 blocks do not; the same with the rotation
+  // epilogue since its stores go through LDS)
+  const bool high = gx * gy * split >= 192 || M <= 64;
   if (!high) gy = ceil_div(M, 64);
   dim3 grid(8 * ceil_div(gx * gy, 8), split);
 #define GO(TMV, XFV) \
@@ -962,8 +1091,9 @@ extern "C" int alice_linear_rope_cache(const void* x, int x_layout, const void* 
   ALICE_CHECK(nH >= 1 && nKV >= 1 && d >= 16 && d % 16 == 0, "linear+rope: bad heads nH=%d nKV=%d d=%d (d must be a multiple of 16)", nH, nKV, d);
   ALICE_CHECK(x && w && q_out && k_pool && v_pool && cos_t && sin_t && positions && seq_of_token && block_table,
               "linear+rope: a pointer is missing");
-  ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)q_out & 3) == 0 && ((uintptr_t)cos_t & 7) == 0 &&
-              ((uintptr_t)sin_t & 7) == 0 && ((uintptr_t)k_pool & 3) == 0, "linear+rope: operands are not aligned");
+  ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)q_out & 15) == 0 && ((uintptr_t)cos_t & 7) == 0 &&
+              ((uintptr_t)sin_t & 7) == 0 && ((uintptr_t)k_pool & 15) == 0 && ((uintptr_t)v_pool & 15) == 0,
+              "linear+rope: operands are not aligned");
   ALICE_CHECK(x_layout == ALICE_LAYOUT_ROW || (x_layout == ALICE_LAYOUT_FRAG16 && K % 32 == 0),
               "linear+rope: activations in fragment order need K %% 32 == 0, found K=%d", K);
   ALICE_CHECK(page_size > 0 && n_pages > 0 && bt_stride > 0, "linear+rope: bad page geometry");

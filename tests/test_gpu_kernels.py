@@ -733,19 +733,29 @@ def test_rope_takes_pairs_next_to_each_other(dt, nH, nKV, d, T, layout):
 
 
 @pytest.mark.parametrize("nH,nKV,d,K", [(8, 4, 256, 2304), (3, 1, 64, 96), (4, 2, 128, 320), (2, 2, 16, 72), (16, 16, 128, 64)])
-@pytest.mark.parametrize("M", [1, 7, 16, 33, 64, 130, 300])
+@pytest.mark.parametrize("M", [1, 7, 16, 33, 64, 130, 300, -300, -3100])
 @pytest.mark.parametrize("layout", [0, 1])
 def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K, M, layout):
     if layout == 1 and d % 32:
         pytest.skip("the fragment cache layout takes head sizes in steps of 32")
+    runs, M = M < 0, abs(M)
+    if M > 1000 and K < 2304:
+        pytest.skip("the longest case once")
     N = (nH + 2 * nKV) * d
     x, w = rnd(M, K, seed=60, dtype=torch.bfloat16), rnd(N, K, seed=61, scale=0.1, dtype=torch.bfloat16)
     wf = ops.to_frag16(w[pair_order(nH, nKV, d).to(DEV)].contiguous())
-    # up to five sequences that start at different places; consecutive tokens go to different sequences
-    n_seq, starts = min(M, 5), [0, 60, 100, 7, 33]
-    order = torch.randperm(n_seq, generator=torch.Generator().manual_seed(1)).tolist()
-    pos = torch.tensor([starts[t % n_seq] + t // n_seq for t in range(M)], dtype=torch.int32, device=DEV)
-    seq = torch.tensor([order[t % n_seq] for t in range(M)], dtype=torch.int32, device=DEV)
+    if runs:
+        # two prompts one after the other: the first starts at place 0, so that its tokens come in whole tiles of
+        # the cache (the kernels' wide stores), the second at place 5 and at a token that is no multiple of 32
+        n_seq, first = 2, (M // 2) // 32 * 32 + 6
+        pos = torch.tensor([t if t < first else 5 + t - first for t in range(M)], dtype=torch.int32, device=DEV)
+        seq = torch.tensor([1 if t < first else 0 for t in range(M)], dtype=torch.int32, device=DEV)
+    else:
+        # up to five sequences that start at different places; consecutive tokens go to different sequences
+        n_seq, starts = min(M, 5), [0, 60, 100, 7, 33]
+        order = torch.randperm(n_seq, generator=torch.Generator().manual_seed(1)).tolist()
+        pos = torch.tensor([starts[t % n_seq] + t // n_seq for t in range(M)], dtype=torch.int32, device=DEV)
+        seq = torch.tensor([order[t % n_seq] for t in range(M)], dtype=torch.int32, device=DEV)
     lens = [int(pos.max()) + 1]
     ang = torch.arange(max(lens), dtype=D)[:, None] * 1e4 ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
     cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
