@@ -50,3 +50,38 @@ def test_real_widths_whole_and_token_by_token(name):
         assert max_err(cut, ref) < TOL[dtype] * scale, (dtype, max_err(cut, ref))
         del model, eng
         torch.cuda.empty_cache()
+
+
+ODD = {
+    # a width that is no multiple of 8, as many groups as heads, a vocabulary of 257
+    "width-100": dict(_COMMON, num_hidden_layers=2, hidden_size=100, num_attention_heads=5, num_key_value_heads=5, head_dim=16,
+                      intermediate_size=136, vocab_size=257, sliding_window=9, query_pre_attn_scalar=16),
+    # a head size that is a multiple of 16 and not of 32, three heads on one group
+    "head-80": dict(_COMMON, num_hidden_layers=2, hidden_size=160, num_attention_heads=6, num_key_value_heads=2, head_dim=80,
+                    intermediate_size=200, vocab_size=300, sliding_window=33, query_pre_attn_scalar=80),
+    # query width three times the width, an odd feed-forward width, a scale that is not the head size
+    "head-96": dict(_COMMON, num_hidden_layers=1, hidden_size=64, num_attention_heads=2, num_key_value_heads=2, head_dim=96,
+                    intermediate_size=17, vocab_size=99, sliding_window=5, query_pre_attn_scalar=7),
+}
+
+
+@pytest.mark.parametrize("name", list(ODD))
+def test_odd_sizes_whole_and_token_by_token(name):
+    """Sizes that fit no tile: every kernel takes them (or hands over to one that does); none gives a wrong result."""
+    folder = os.path.join(_TMP.name, name)
+    alice.write_random_model(folder, dict(ODD[name]), seed=4)
+    plain = plain_model(folder)
+    toks = random_tokens(plain.V, 90, 61)
+    ref = plain.forward(toks)
+    scale = max(1.0, float(ref.abs().max()))
+    for dtype in ("float32", "bfloat16"):
+        model = alice.load(folder, dtype=dtype)
+        eng = model.engine(max_tokens=256, max_seqs=2)
+        s = eng.open(1)
+        whole = eng.step(s, [toks], "all")
+        eng.close(s)
+        s = eng.open(1)
+        cut = [eng.step(s, [toks[:70]], "all")] + [eng.step(s, [[t]], "last") for t in toks[70:]]
+        eng.close(s)
+        assert max_err(whole, ref) < TOL[dtype] * scale, (dtype, max_err(whole, ref))
+        assert max_err(torch.cat(cut), ref) < TOL[dtype] * scale, (dtype, max_err(torch.cat(cut), ref))
