@@ -81,17 +81,25 @@ struct Core {
 
   // The fragments of one block of 32 keys: kpage/vpage point at the page of one kv head, kb is the block
   // within the page (0/1).
+  // ONCE: the tile is read once per step by one wave (single tokens): loaded with the streaming hint.
+  template <bool ONCE = false>
+  __device__ __forceinline__ static u32x4 load_tile(const bf16_t* p) {
+    if constexpr (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    else return *reinterpret_cast<const u32x4*>(p);
+  }
+  template <bool ONCE = false>
   __device__ __forceinline__ static void load_k(const bf16_t* __restrict__ kpage, int kb, int lane, u32x4 (&kf)[2][DT]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
-        kf[t][dt] = *reinterpret_cast<const u32x4*>(kpage + ((size_t)((kb * 2 + t) * DT + dt) * 64 + lane) * 8);
+        kf[t][dt] = load_tile<ONCE>(kpage + ((size_t)((kb * 2 + t) * DT + dt) * 64 + lane) * 8);
   }
+  template <bool ONCE = false>
   __device__ __forceinline__ static void load_v(const bf16_t* __restrict__ vpage, int kb, int lane, u32x4 (&vf)[2 * DT]) {
 #pragma unroll
     for (int t = 0; t < 2 * DT; ++t)
-      vf[t] = *reinterpret_cast<const u32x4*>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
+      vf[t] = load_tile<ONCE>(vpage + ((size_t)(kb * 2 * DT + t) * 64 + lane) * 8);
   }
 
   // Scores of one block of 32 keys from loaded key fragments; key0 is the absolute position of its first
@@ -606,8 +614,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     u32x4 kf0[2][DT], vf0[2 * DT], kf1[2][DT], vf1[2 * DT];
     auto page_of = [&](int kb32) { return bt[min(kb32, my_last) >> 1]; };
     auto fetch = [&](int kb32, int page, u32x4 (&kf)[2][DT], u32x4 (&vf)[2 * DT]) {
-      Core<DT, 1>::load_k(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
-      Core<DT, 1>::load_v(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
+      Core<DT, 1>::template load_k<true>(k_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, kf);
+      Core<DT, 1>::template load_v<true>(v_pool + ((size_t)page * nKV + kvh) * page_elems, kb32 & 1, lane, vf);
     };
     int page_a = 0, page_b = 0;
     if (my_first <= my_last) {

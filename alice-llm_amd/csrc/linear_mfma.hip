@@ -241,8 +241,15 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
   auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
     const bool kok = kt < ke;
     const int ktc = kok ? kt : 0;                           // past the slice: zero weights, any activations
+    // The tallest matrices (the output head: hundreds of MB at up to 16 tokens) are read with the streaming hint:
+    // 6.5 against 5.85 TB/s at the 2B head.  The layers' matrices are not: the same hint cost the down projection
+    // 8 % and changed the others by 2 % either way.
 #pragma unroll
-    for (int i = 0; i < RT; ++i) aa[i] = *reinterpret_cast<const u32x4*>(kok ? wrow[i] + (size_t)ktc * 512 : zero);
+    for (int i = 0; i < RT; ++i) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(kok ? wrow[i] + (size_t)ktc * 512 : zero);
+      if constexpr (RT == 4 && MT == 1) aa[i] = __builtin_nontemporal_load(src);
+      else aa[i] = *src;
+    }
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       if constexpr (XF) {
