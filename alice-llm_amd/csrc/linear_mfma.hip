@@ -196,7 +196,7 @@ __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const Rop
 // valid ones and what they bring is replaced by zeros (weights) or lands in output columns that are never
 // stored (tokens beyond M).  Only then does the compiler know how many loads are in flight and wait for the
 // oldest alone (s_waitcnt vmcnt(n)); a load under a branch makes it wait for all of them.
-template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF>
+template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF, bool STREAM = false>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
                                                             int kt_per_slice, float epi, int y_frag, RopeArgs ra) {
@@ -241,13 +241,13 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
   auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
     const bool kok = kt < ke;
     const int ktc = kok ? kt : 0;                           // past the slice: zero weights, any activations
-    // The tallest matrices (the output head: hundreds of MB at up to 16 tokens) are read with the streaming hint:
-    // 6.5 against 5.85 TB/s at the 2B head.  The layers' matrices are not: the same hint cost the down projection
-    // 8 % and changed the others by 2 % either way.
+    // STREAM: a matrix of 96 MB or more is read with the streaming hint (the 2B output head: 6.5 against 5.85 TB/s;
+    // the 9B and 27B layers' matrices: 4 to 7 % faster).  Smaller ones are not: the hint cost the 2B down
+    // projection (42 MB) 8 % and changed the others by 2 % either way.
 #pragma unroll
     for (int i = 0; i < RT; ++i) {
       const u32x4* src = reinterpret_cast<const u32x4*>(kok ? wrow[i] + (size_t)ktc * 512 : zero);
-      if constexpr (RT == 4 && MT == 1) aa[i] = __builtin_nontemporal_load(src);
+      if constexpr (STREAM) aa[i] = __builtin_nontemporal_load(src);
       else aa[i] = *src;
     }
 #pragma unroll
@@ -904,13 +904,16 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   // Eight waves a block when the slice is long enough to give each of them work and the block count is
   // too low to fill the chip with four.
   const bool eight = (RT * MT <= 4) && per >= 32 && groups * split < 2048;
+  const bool stream_w = x_frag && (size_t)NT * KT * 1024 >= ((size_t)96 << 20);
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
-    if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    if (stream_w) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    else if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
     else linear_skinny_kernel<RT, MT, 8, EPI, TO, false, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
   } else {
     const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-    if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    if (stream_w) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    else if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
     else linear_skinny_kernel<RT, MT, 4, EPI, TO, false, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
   }
   ALICE_LAUNCH_CHECK();
