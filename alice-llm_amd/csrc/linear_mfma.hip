@@ -1064,8 +1064,9 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
               "linear: activations in fragment order need K %% 32 == 0, found K=%d", K);
   if (M == 0) return 0;
   // Up to 64 tokens stream the weights once; very wide matrices (the output head) have enough column
-  // blocks for the tiled kernel, which shares the activations through LDS, as soon as there are 17 tokens.
-  bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 16 && N >= 65536 && split_k == 1));
+  // blocks for the tiled kernel, which shares the activations through LDS, from 33 tokens on (the 2B head: the same
+  // time at 32 tokens, 228 against 277 us at 48; the streaming kernel 198 against 210 us at 17).
+  bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 32 && N >= 65536 && split_k == 1));
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
   ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),
               "linear: partial sums need no epilogue and float32 output");
