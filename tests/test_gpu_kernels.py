@@ -500,6 +500,29 @@ def test_linear_mfma_geglu(M, N, K):
         close(y, ref, 2e-2, 2 ** -7)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 24])
+def test_linear_mfma_matrices_read_with_the_streaming_hint(M):
+    """Matrices of 96 MB or more are read by the streaming kernel with the streaming hint (another instantiation of
+    the kernel): the same sums as the tiled kernel, which reads them plainly, and as the plain product."""
+    N, K = 26000, 2048                                       # 106 MB in bfloat16
+    g = torch.Generator(device=DEV).manual_seed(5)
+    w = (torch.randn(N, K, generator=g, device=DEV) * 0.1).to(torch.bfloat16)
+    x = rnd(M, K, seed=6, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    ref = (x.double() @ w.double().T).cpu()
+    for epi, param, want in ((ops.EPI_NONE, 0.0, ref), (ops.EPI_SOFTCAP, 3.0, 3.0 * torch.tanh(ref / 3.0))):
+        ys = []
+        for variant in (ops.LINEAR_SKINNY, ops.LINEAR_MFMA):
+            for frag_in in (True, False):
+                y = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+                ops.linear(acts_to_fragments(x) if frag_in else x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=epi,
+                           epi_param=param, variant=variant, full_precision=False, rows=M,
+                           x_layout=ops.LAYOUT_FRAG16 if frag_in else ops.LAYOUT_ROW)
+                close(y, want, 1e-3, 1e-5)
+                ys.append(y)
+        assert torch.equal(ys[0], ys[1])                     # with the hint (fragments in) and without (rows in)
+
+
 def test_linear_mfma_rows_do_not_depend_on_the_batch():
     # a token's output is the same whatever else is in the batch, within each kernel
     x, w = rnd(64, 320, seed=20, dtype=torch.bfloat16), rnd(208, 320, seed=21, scale=0.1, dtype=torch.bfloat16)
