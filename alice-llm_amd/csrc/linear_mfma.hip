@@ -503,8 +503,8 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
 
   if constexpr (EPI == ALICE_EPI_ROPE) {
     // The rotated values go to their places through LDS, 64 tokens at a time: a lane holds two pairs of a token
-    // (4-byte pieces of 16 different rows of q or of the cache), and stores of such pieces cost several times the
-    // product's own time per byte.  Staged, a token's 16 features of a weight tile become two runs of eight
+    // (4-byte pieces of 16 different rows of q or of the cache), eight such stores per token tile and wave (measured:
+    // 4 to 6 % of the kernel against the staging below).  Staged, a token's 16 features of a weight tile become two runs of eight
     // neighbouring elements of a head (the low and the high halves of eight pairs; a value head's 16 elements as
     // they are), and every thread then moves 16-byte runs: along a token for q and for row-major caches, along 16
     // tokens for keys in fragment order (a 1 KB tile per wave when the tokens start at a multiple of 16), and for
