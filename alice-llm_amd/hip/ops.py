@@ -411,11 +411,18 @@ def attention_mfma_supported(head_dim: int) -> bool:
 
 
 def decode_splits(n_seqs: int, num_kv_heads: int, max_context: int) -> int:
-    """Into how many blocks the keys of a sequence are split for single-token attention: enough to
-    fill the chip (about a thousand waves), at least eight 32-key blocks per block of four waves."""
-    by_fill = -(-1024 // max(1, n_seqs * num_kv_heads * 4))
-    by_work = max(1, -(-max_context // 32) // 8)
-    return max(1, min(by_fill, by_work, 64))
+    """Into how many blocks the keys of a sequence are split for single-token attention.  At most as many as fill
+    the chip (about a thousand waves); among those, the fewest that leave a wave the fewest 32-key blocks to walk
+    through one after the other, but no fewer than two (125 blocks of keys: 16 splits of four waves walk two each,
+    15 splits three)."""
+    n_blocks = -(-max_context // 32)
+    cap = max(1, min(-(-1024 // max(1, n_seqs * num_kv_heads * 4)), 64))
+    best, best_per = 1, -(-n_blocks // 4)
+    for s in range(2, cap + 1):
+        per = -(-n_blocks // (4 * s))
+        if 2 <= per < best_per:
+            best, best_per = s, per
+    return best
 
 
 PREFILL_AUTO, PREFILL_TILES, PREFILL_SPLIT, PREFILL_SHARED4, PREFILL_SHARED8, PREFILL_SHARED4X2 = 0, 1, 2, 3, 4, 5
