@@ -235,7 +235,10 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
   // A rolling window of U k-tiles per wave: wave w takes k-tiles kb + w, kb + w + NW, ...; as soon as a
   // tile's fragments have gone into the MFMAs their registers are refilled with the tile U steps ahead,
   // so U loads per operand stay in flight all the time.
-  constexpr int U = (RT * MT >= 8) ? 3 : 4;
+  // (Five for one or two products per k-tile: the layers' matrices at up to 16 tokens give a wave 9 k-tiles, which are
+  // two windows of five with one idle slot instead of three of four with three, or 5, which is one window and no loop:
+  // a 2B layer's six kernels 54.0 -> 51.9 us; six and eight were slower.)
+  constexpr int U = (RT * MT >= 8) ? 3 : (RT * MT <= 2 ? 5 : 4);
   u32x4 a[U][RT], b[U][MT];
   const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
   auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
