@@ -196,7 +196,7 @@ __device__ __forceinline__ void rope_store4(const RopeArgs& ra, int m, const Rop
 // valid ones and what they bring is replaced by zeros (weights) or lands in output columns that are never
 // stored (tokens beyond M).  Only then does the compiler know how many loads are in flight and wait for the
 // oldest alone (s_waitcnt vmcnt(n)); a load under a branch makes it wait for all of them.
-template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF, bool STREAM = false>
+template <int RT, int MT, int NW, int EPI, typename TO, bool FULL, bool XF, bool STREAM = false, int WINDOW = 0>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
                                                             TO* __restrict__ y, int M, int N, int K, int KT, int NT,
                                                             int kt_per_slice, float epi, int y_frag, RopeArgs ra) {
@@ -235,10 +235,12 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
   // A rolling window of U k-tiles per wave: wave w takes k-tiles kb + w, kb + w + NW, ...; as soon as a
   // tile's fragments have gone into the MFMAs their registers are refilled with the tile U steps ahead,
   // so U loads per operand stay in flight all the time.
-  // (Five for one or two products per k-tile: the layers' matrices at up to 16 tokens give a wave 9 k-tiles, which are
-  // two windows of five with one idle slot instead of three of four with three, or 5, which is one window and no loop:
-  // a 2B layer's six kernels 54.0 -> 51.9 us; six and eight were slower.)
-  constexpr int U = (RT * MT >= 8) ? 3 : (RT * MT <= 2 ? 5 : 4);
+  // The window is 4 (3 with eight or more products per k-tile), or 5 where the launcher finds that this leaves fewer
+  // idle slots in a wave's last window (WINDOW; one or two products per k-tile only): 9 k-tiles a wave are two windows
+  // of five with one idle slot instead of three of four with three, and 5 k-tiles one window and no loop (a 2B layer's
+  // six kernels 54.0 -> 51.9 us), while 7 k-tiles are better off with two windows of four (9B down projection: 22.3
+  // against 25.0 us).  Six and eight were slower everywhere.
+  constexpr int U = WINDOW > 0 ? WINDOW : ((RT * MT >= 8) ? 3 : 4);
   u32x4 a[U][RT], b[U][MT];
   const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
   auto fetch = [&](int kt, u32x4 (&aa)[RT], u32x4 (&bb)[MT]) {
@@ -908,17 +910,31 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   // too low to fill the chip with four.
   const bool eight = (RT * MT <= 4) && per >= 32 && groups * split < 2048;
   const bool stream_w = x_frag && (size_t)NT * KT * 1024 >= ((size_t)96 << 20);
+  // k-tiles per wave, and whether windows of five waste fewer slots than windows of four (see the kernel)
+  const int nw = eight ? 8 : 4, J = ceil_div(min(per, KT), nw);
+  const bool five = RT * MT <= 2 && x_frag && (ceil_div(J, 5) * 5 - J) < (ceil_div(J, 4) * 4 - J);
+#define SKINNY(NWV, THREADS, XFV, STREAMV, WINV)                                                                             \
+  linear_skinny_kernel<RT, MT, NWV, EPI, TO, false, XFV, STREAMV, WINV><<<grid, THREADS, lds, s>>>(                           \
+      (const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra)
+#define BY_INPUT(NWV, THREADS)                                                        \
+  do {                                                                                \
+    if constexpr (RT * MT <= 2) {                                                     \
+      if (five && stream_w) { SKINNY(NWV, THREADS, true, true, 5); break; }           \
+      if (five) { SKINNY(NWV, THREADS, true, false, 5); break; }                      \
+    }                                                                                 \
+    if (stream_w) SKINNY(NWV, THREADS, true, true, 0);                                \
+    else if (x_frag) SKINNY(NWV, THREADS, true, false, 0);                            \
+    else SKINNY(NWV, THREADS, false, false, 0);                                       \
+  } while (0)
   if (eight) {
     const size_t lds = (size_t)7 * RT * MT * 256 * sizeof(float);
-    if (stream_w) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
-    else if (x_frag) linear_skinny_kernel<RT, MT, 8, EPI, TO, false, true><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
-    else linear_skinny_kernel<RT, MT, 8, EPI, TO, false, false><<<grid, 512, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    BY_INPUT(8, 512);
   } else {
     const size_t lds = (size_t)3 * RT * MT * 256 * sizeof(float);
-    if (stream_w) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
-    else if (x_frag) linear_skinny_kernel<RT, MT, 4, EPI, TO, false, true><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
-    else linear_skinny_kernel<RT, MT, 4, EPI, TO, false, false><<<grid, 256, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);
+    BY_INPUT(4, 256);
   }
+#undef BY_INPUT
+#undef SKINNY
   ALICE_LAUNCH_CHECK();
   return 0;
 }
