@@ -1,9 +1,11 @@
-"""Import name of the package whose sources live in the folder `alice-llm_amd/` (a hyphen cannot be
-imported): this module points its search path there and runs that folder's __init__."""
-import os as _os
-
-_real = _os.path.join(_os.path.dirname(_os.path.dirname(_os.path.abspath(__file__))), "alice-llm_amd")
-__path__[:] = [_real]
-with open(_os.path.join(_real, "__init__.py")) as _f:
-    exec(compile(_f.read(), _os.path.join(_real, "__init__.py"), "exec"))
-del _f
+"""alice-llm_amd: a small Gemma 2 library for one MI355X: configuration and registry, safetensors
+weights, layers built from parts, a paged cache with slots, one step function, a generation loop
+with sampling, and hand-written HIP kernels for gfx950 in bfloat16 and in true 32-bit."""
+from .config import (ConfigError, Gemma2Config, config_from_dict, load_config, register_architecture,
+                     registered_architectures)
+from .config.presets import preset, preset_names
+from .parts import Precision
+from .weights.loader import WeightError, init_random, load_weights, write_random_model
+from .weights.safetensors_io import WeightFileError
+from .cache import Cache, CacheError
+from .api import Model, load, GenerationResult
