@@ -5,7 +5,10 @@ from .config import (ConfigError, Gemma2Config, config_from_dict, load_config, r
                      registered_architectures)
 from .config.presets import preset, preset_names
 from .parts import Precision
-from .weights.loader import WeightError, init_random, load_weights, write_random_model
+from .weights.loader import UnexpectedTensorsWarning, WeightError, init_random, load_weights, write_random_model
 from .weights.safetensors_io import WeightFileError
 from .cache import Cache, CacheError
-from .api import Model, load, GenerationResult
+from .api import Model, load, sample, GenerationResult
+from .engine.step import Engine
+from .engine.generate import Generator
+from .sampling import Sampler

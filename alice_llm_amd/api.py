@@ -29,13 +29,14 @@ class Model:
 
     # ------------------------------------------------------------------ construction
     @classmethod
-    def load(cls, folder: str, dtype=None, device: Union[str, torch.device, None] = None) -> "Model":
-        """A folder with config.json and model.safetensors; the model class is chosen by config.json."""
+    def load(cls, folder: str, dtype=None, device: Union[str, torch.device, None] = None, strict: bool = True) -> "Model":
+        """A folder with config.json and model.safetensors; the model class is chosen by config.json.
+        strict=False: tensors in the folder that the model does not declare are warned about, not an error."""
         config = load_config(folder)
         device = torch.device(device) if device is not None else ops.require_gpu()
         precision = Precision.of(dtype or getattr(config, "torch_dtype", "bfloat16"))
         lm = CausalLM(config.plan(), precision, device)
-        load_weights(lm, folder)
+        load_weights(lm, folder, strict)
         return cls(config, lm)
 
     @classmethod
@@ -54,35 +55,69 @@ class Model:
         return cls(config, lm)
 
     # ------------------------------------------------------------------ use
-    def engine(self, max_tokens: int, max_seqs: Optional[int] = None, use_graphs: Optional[bool] = None) -> Engine:
-        """A cache sized for max_tokens and the step function over it.  use_graphs: record decode steps into
-        HIP graphs (default: whenever every part of the model allows it)."""
-        return Engine(self.lm, max_tokens=max_tokens, max_seqs=max_seqs, use_graphs=use_graphs)
+    def engine(self, max_tokens: Optional[int] = None, max_seqs: Optional[int] = None,
+               use_graphs: Optional[bool] = None, *, seq_lens: Optional[Sequence[int]] = None, **kw) -> Engine:
+        """A cache and the step function over it.  The cache is sized for max_tokens (each live sequence's count
+        rounded up to whole pages) or for sequences of the lengths `seq_lens` held together.  use_graphs: record
+        decode steps into HIP graphs (default: whenever every part of the model allows it)."""
+        return Engine(self.lm, max_tokens=max_tokens, seq_lens=seq_lens, max_seqs=max_seqs, use_graphs=use_graphs, **kw)
 
     new_cache = engine
+
+    def step(self, engine: Engine, slots: Sequence[int], new_tokens: Sequence[Sequence[int]], want="last") -> torch.Tensor:
+        """One step of `engine` (made by this model's engine()): new_tokens[i] for the sequence in slots[i]; float32
+        logits at the wanted places.  The same as engine.step; the reference's Llama3Model::forward (llama3.rs:13496)."""
+        if engine.model is not self.lm:
+            raise ValueError("this engine belongs to another model")
+        return engine.step(slots, new_tokens, want)
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: Union[int, Sequence[int]] = 256,
                  temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
                  stop_token_ids: Optional[Sequence[int]] = None, max_batch: Optional[int] = None,
-                 max_tokens: Optional[int] = None, engine: Optional[Engine] = None) -> List[GenerationResult]:
-        """Generate for every prompt (token ids); as many batches one after another as needed."""
+                 max_tokens: Optional[int] = None, engine: Optional[Engine] = None,
+                 observer=None) -> List[GenerationResult]:
+        """Generate for every prompt (token ids); as many batches one after another as needed.  A request whose
+        prompt and cap together outgrow the model's positions ends at the last position with finish_reason
+        "length".  observer: see Generator."""
         if prompts and isinstance(prompts[0], int):
             prompts = [prompts]
         caps = [max_new_tokens] * len(prompts) if isinstance(max_new_tokens, int) else list(max_new_tokens)
         if engine is None:
             batch = max_batch or len(prompts)
-            longest = sorted((len(p) + c for p, c in zip(prompts, caps)), reverse=True)[:batch]
-            need = sum(-(-n // 64) * 64 for n in longest)
-            engine = self.engine(max_tokens or need, max_seqs=batch)
+            most = self.lm.plan.max_positions
+            longest = sorted((min(len(p) + max(c - 1, 0), most) for p, c in zip(prompts, caps)), reverse=True)[:batch]
+            engine = (self.engine(max_tokens, max_seqs=batch) if max_tokens else
+                      self.engine(seq_lens=longest, max_seqs=batch))
         if stop_token_ids is None:
             stop_token_ids = self.lm.plan.stop_token_ids
         gen = Generator(engine, temperature=temperature, top_k=top_k, top_p=top_p, seed=seed,
-                        stop_token_ids=stop_token_ids, max_batch=max_batch)
+                        stop_token_ids=stop_token_ids, max_batch=max_batch, observer=observer)
         return gen.run(prompts, caps)
 
 
-def load(path_or_config, dtype=None, random_seed: Optional[int] = None, device=None) -> Model:
+def sample(logits: torch.Tensor, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, u=None) -> torch.Tensor:
+    """One token id per row of float32 logits [rows, vocab] (or one row [vocab]) on the GPU, as int32 [rows]:
+    temperature, then top-k, then top-p, then softmax, then the inverse CDF at u[row] in [0, 1)
+    (src/sampling.rs:10-123; the order of examples/generate_gpu.rs:125-128).  A temperature below 1e-6 is greedy,
+    the lowest index among equal maxima, and needs no u."""
+    from .sampling import GREEDY_BELOW
+    if logits.dim() == 1:
+        logits = logits[None]
+    logits = logits.contiguous()
+    if temperature < GREEDY_BELOW:
+        return ops.argmax(logits)
+    if u is None:
+        raise ValueError("sampling at a temperature needs u: one uniform number in [0, 1) per row")
+    u = torch.as_tensor(u, dtype=torch.float32).reshape(-1).to(logits.device)
+    if u.numel() != logits.shape[0] or bool(((u < 0) | (u >= 1)).any()):
+        raise ValueError("u must hold one number in [0, 1) per row of logits")
+    if top_k < 0 or not top_p > 0:
+        raise ValueError("top_k must not be negative and top_p must be positive")
+    return ops.sample(logits, u, float(temperature), int(top_k), float(top_p))
+
+
+def load(path_or_config, dtype=None, random_seed: Optional[int] = None, device=None, strict: bool = True) -> Model:
     """load("folder") reads a model folder; load(config_dict_or_object, random_seed=0) makes random weights."""
     if isinstance(path_or_config, (str, os.PathLike)):
-        return Model.load(os.fspath(path_or_config), dtype, device)
+        return Model.load(os.fspath(path_or_config), dtype, device, strict)
     return Model.random(path_or_config, random_seed or 0, dtype, device)

@@ -76,9 +76,12 @@ class PageGroup:
         self.n_pages = n_pages                      # usable pages; page 0 of the pool is never handed out
         self._free: List[int] = list(range(n_pages, 0, -1))
         self._table: Dict[int, List[int]] = {}      # slot -> page id per page index, -1 once given back
-        shape = (len(self.layers), n_pages + 1, need.num_kv_heads, page_size, need.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
-        self.v = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
+        if need.page_size is not None and need.page_size != page_size:
+            raise CacheError(f"the layers {self.layers} need pages of {need.page_size} positions (their kernels are "
+                             f"written for that), the cache has pages of {page_size}")
+        shape = (len(self.layers), n_pages + 1, need.num_kv_heads, page_size)
+        self.k = torch.zeros(shape + (need.head_dim,), dtype=dtype, device=device) if allocate else None
+        self.v = torch.zeros(shape + (need.v_dim,), dtype=dtype, device=device) if allocate else None
 
     # -- bookkeeping (host only) ---------------------------------------------------------
     def open(self, slot: int) -> None:
@@ -137,7 +140,7 @@ class LayerCache:
     v: Optional[torch.Tensor]
     block_table: Optional[torch.Tensor]   # int32 [sequences of the step, pages]
     writable: bool                        # False when the run reads another layer's cache
-    state: Optional[torch.Tensor]         # [slots, *shape]: index with ctx.slots
+    state: Dict[str, torch.Tensor]        # by the name of its StateNeed: [slots + 1, *shape], index with ctx.slots
     group: Optional[int] = None
 
 
@@ -163,18 +166,23 @@ class Cache:
         for gi, g in enumerate(self.groups):
             for li, layer in enumerate(g.layers):
                 self._where[layer] = (gi, li)
-        self.state: Dict[int, torch.Tensor] = {}
+        # Fixed-size state: per run of the schedule, one tensor per declared StateNeed with a row per slot and one
+        # spare row (index n_slots) that the padded rows of a captured decode step read and write.
+        self.spare_slot = n_slots
+        self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         for i, need in enumerate(needs):
-            if need is not None and need.state is not None and allocate:
-                self.state[i] = torch.zeros((n_slots, *need.state.shape), dtype=need.state.dtype, device=device)
+            if need is not None and need.state and allocate:
+                self.state[i] = {st.name: torch.zeros((n_slots + 1, *st.shape), dtype=st.dtype, device=device)
+                                 for st in need.state}
 
     # -- slots ---------------------------------------------------------------------------
     def open(self) -> int:
         slot = self.slots.take()
         for g in self.groups:
             g.open(slot)
-        for t in self.state.values():
-            t[slot].zero_()
+        for tensors in self.state.values():
+            for t in tensors.values():
+                t[slot].zero_()
         return slot
 
     def close(self, slot: int) -> None:
@@ -248,7 +256,7 @@ class Cache:
             gi, li = self._where[src]
             k, v, bt = self.groups[gi].k[li], self.groups[gi].v[li], block_tables[gi]
         return LayerCache(k=k, v=v, block_table=bt, writable=read_from is None,
-                          state=self.state.get(src), group=gi)
+                          state=self.state.get(src, {}), group=gi)
 
     def check_consistent(self) -> None:
         """No page lost, held twice, or both free and held (for tests)."""

@@ -53,6 +53,12 @@ class Gemma2Config:
         require(nH > 0, "num_attention_heads must be positive")
         hd = read_key(d, "head_dim", int, H // nH)
         I = read_key(d, "intermediate_size", int)
+        # Keys that would change the arithmetic and that nothing here implements are refused, not dropped: the
+        # projections have no biases (llama3.rs:14206-14217: the bias branches are no-ops for this architecture)
+        # and the rotation has no scaling factors (no rope_freqs tensor, llama3.rs:5367-5378).
+        require(not read_key(d, "attention_bias", bool, False),
+                "attention_bias is true, and the attention projections here have no biases")
+        require(d.get("rope_scaling") is None, f"rope_scaling {d.get('rope_scaling')!r} is not implemented (null only)")
         eos = d.get("eos_token_id", 1)
         if isinstance(eos, int) and not isinstance(eos, bool):
             eos = (eos,)

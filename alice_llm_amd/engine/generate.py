@@ -12,8 +12,6 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence
 
-PAGE = 64
-
 
 @dataclass
 class GenerationResult:
@@ -28,8 +26,24 @@ class GenerationResult:
         return len(self.tokens)
 
 
+def limit_caps(prompt_lens: Sequence[int], caps: Sequence[int], max_positions: Optional[int]) -> List[int]:
+    """Each request's cap of new tokens, cut so that the sequence never outgrows max_positions: a prompt of n
+    tokens can draw max_positions - n + 1 tokens (the last one drawn is never fed back).  The reference ends
+    such a sequence at its cap, not the whole call (llama3.rs:17813-17835).  A prompt that is itself longer than
+    max_positions is an error, raised before anything runs, that names the request."""
+    if max_positions is None:
+        return [max(int(c), 0) for c in caps]
+    out = []
+    for i, (n, c) in enumerate(zip(prompt_lens, caps)):
+        if n > max_positions:
+            raise ValueError(f"request {i}: its prompt of {n} tokens is longer than the model's "
+                             f"{max_positions} positions")
+        out.append(max(0, min(int(c), max_positions - n + 1)))
+    return out
+
+
 def plan_batches(prompt_lens: Sequence[int], caps: Sequence[int], *, max_batch: Optional[int],
-                 capacity_tokens: int, max_slots: int, page: int = PAGE) -> List[List[int]]:
+                 capacity_tokens: int, max_slots: int, page: int) -> List[List[int]]:
     """Split requests, in order, into batches that fit: at most max_batch (and max_slots) sequences,
     and room in the cache for every sequence at its longest, each rounded up to whole pages."""
     limit = min(max_batch or max_slots, max_slots)
@@ -37,7 +51,7 @@ def plan_batches(prompt_lens: Sequence[int], caps: Sequence[int], *, max_batch: 
     cur: List[int] = []
     used = 0
     for i, (n, c) in enumerate(zip(prompt_lens, caps)):
-        need = -(-(n + max(c, 0)) // page) * page
+        need = -(-(n + max(c - 1, 0)) // page) * page         # the last token drawn is not fed back
         if need > capacity_tokens:
             raise ValueError(f"request {i} needs room for {need} tokens, the cache holds {capacity_tokens}")
         if cur and (len(cur) >= limit or used + need > capacity_tokens):
@@ -57,7 +71,11 @@ class Generator:
 
     def __init__(self, engine, *, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
                  stop_token_ids: Sequence[int] = (), max_batch: Optional[int] = None,
-                 sampler: Optional[Callable] = None, include_stop_token: bool = False):
+                 sampler: Optional[Callable] = None, include_stop_token: bool = False,
+                 observer: Optional[Callable] = None):
+        """observer(requests, positions, logits, tokens), if given, is called after every step of every batch
+        with the live requests' indices, the position each row's logits belong to, the step's float32 logits
+        [rows, vocab] and the token ids drawn from them: what a logits dump of the real run needs."""
         self.engine = engine
         if sampler is None:
             from ..sampling import Sampler
@@ -66,6 +84,7 @@ class Generator:
         self.stop = set(int(t) for t in stop_token_ids)
         self.max_batch = max_batch
         self.include_stop_token = include_stop_token
+        self.observer = observer
 
     def run(self, prompts: Sequence[Sequence[int]], max_new_tokens: Sequence[int]) -> List[GenerationResult]:
         if len(prompts) != len(max_new_tokens):
@@ -74,10 +93,13 @@ class Generator:
             raise ValueError("every prompt needs at least one token")
         results: List[Optional[GenerationResult]] = [None] * len(prompts)
         cache = self.engine.cache
-        batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch=self.max_batch,
-                               capacity_tokens=cache.max_tokens, max_slots=cache.slots.n_slots)
+        lens = [len(p) for p in prompts]
+        # everything that can be refused is refused here, before a slot is taken or a kernel runs
+        caps = limit_caps(lens, max_new_tokens, getattr(self.engine, "max_positions", None))
+        batches = plan_batches(lens, caps, max_batch=self.max_batch, capacity_tokens=cache.max_tokens,
+                               max_slots=cache.slots.n_slots, page=cache.page_size)
         for batch in batches:
-            self._run_batch(batch, prompts, max_new_tokens, results)
+            self._run_batch(batch, prompts, caps, results)
         return results  # type: ignore[return-value]
 
     def _run_batch(self, batch, prompts, caps, results) -> None:
@@ -97,6 +119,8 @@ class Generator:
             while live:
                 logits = eng.step([slots[r] for r in live], feed, "last")
                 ids = self.sampler(logits, live, [len(out[r]) for r in live]).tolist()   # waits for the step
+                if self.observer is not None:
+                    self.observer(list(live), [len(prompts[r]) + len(out[r]) - 1 for r in live], logits, ids)
                 if first:
                     prefill_ms = (time.perf_counter() - t0) * 1e3
                     first = False

@@ -51,7 +51,7 @@ class CausalLM:
                                      f"an earlier entry with a cache of its own")
                 a, b = self._need(e.layer), self._need(plan.schedule[e.cache_from].layer)
                 if a is None or b is None or a.kv is None or b.kv is None or \
-                        (a.kv.num_kv_heads, a.kv.head_dim) != (b.kv.num_kv_heads, b.kv.head_dim) or \
+                        (a.kv.num_kv_heads, a.kv.head_dim, a.kv.v_dim) != (b.kv.num_kv_heads, b.kv.head_dim, b.kv.v_dim) or \
                         (b.kv.window is not None and (a.kv.window is None or a.kv.window > b.kv.window)):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_from}: "
                                      f"its keys differ in shape or reach further back than that cache keeps")

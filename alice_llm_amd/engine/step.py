@@ -16,7 +16,7 @@ from typing import List, Optional, Sequence, Union
 import numpy as np
 import torch
 
-from ..cache import Cache, CacheError
+from ..cache import Cache, CacheError, PAGE_SIZE
 from ..hip import ops
 from .model import CausalLM
 
@@ -37,7 +37,9 @@ class StepContext:
     max_new: int                    # most new tokens of one sequence
     max_context: int                # most keys of one sequence after the step
     max_position: int               # largest position in the step
-    # host copies, for parts that plan their launches
+    # host copies, for parts that plan their launches on the host.  In a captured step (`captured`) they are
+    # placeholders: a part that declares graph_safe reads the device arrays above instead.
+    captured: bool = False
     new_lens: Sequence[int] = ()
     start_lens: Sequence[int] = ()
     slot_ids: Sequence[int] = ()
@@ -119,7 +121,7 @@ class _DecodeGraph:
         self.ctx = StepContext(tokens=part(0), positions=part(1), seq_of_token=part(2), slots=part(3), want_rows=part(4),
                                cu_seqlens=part(5), context_lens=part(6), n_tokens=B, n_seqs=B, is_decode=True,
                                max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
-                               start_lens=[0] * B, slot_ids=[0] * B,
+                               captured=True, start_lens=[0] * B, slot_ids=[0] * B,
                                fragment_activations=engine.model.precision.act == torch.bfloat16,
                                want_every_row=True)
         o = self.offs
@@ -146,6 +148,8 @@ class _DecodeGraph:
         sh[o[0] + n:o[1]] = 0
         sh[o[1]:o[1] + n] = start
         sh[o[1] + n:o[2]] = 0
+        sh[o[3]:o[3] + n] = slots
+        sh[o[3] + n:o[4]] = engine.cache.spare_slot          # padded rows: state of their own that nobody reads
         ctx_lens = sh[o[6]:o[7]]
         ctx_lens[:n] = start
         ctx_lens[:n] += 1
@@ -162,18 +166,28 @@ class _DecodeGraph:
 class Engine:
     """A model, its cache, and the step function over them."""
 
-    def __init__(self, model: CausalLM, *, max_tokens: int, max_seqs: Optional[int] = None,
-                 use_graphs: Optional[bool] = None, max_graphs: int = 24):
+    def __init__(self, model: CausalLM, *, max_tokens: Optional[int] = None, seq_lens: Optional[Sequence[int]] = None,
+                 max_seqs: Optional[int] = None, use_graphs: Optional[bool] = None, max_graphs: int = 24,
+                 page_size: int = PAGE_SIZE):
+        """The cache holds `max_tokens` tokens (each live sequence's count rounded up to whole pages), or, given
+        `seq_lens` instead, room for sequences of these lengths at the same time."""
         self.model = model
         self.device = model.device
         ops.require_gpu()
+        if (max_tokens is None) == (seq_lens is None):
+            raise ValueError("give either max_tokens or seq_lens")
+        if max_tokens is None:
+            max_tokens = sum(-(-int(n) // page_size) * page_size for n in seq_lens)
+            if max_seqs is None:
+                max_seqs = len(seq_lens)
         self.cache = Cache(model.cache_needs(), max_tokens=max_tokens, dtype=model.precision.act,
-                           device=self.device, max_seqs=max_seqs)
+                           device=self.device, max_seqs=max_seqs, page_size=page_size)
         self.vocab_size = model.plan.vocab_size
         self.max_positions = model.plan.max_positions
-        # Decode steps are captured into HIP graphs when every part says its launches can be recorded
-        # (parts that loop on the host over sequences cannot) and no layer keeps fixed-size state.
-        safe = model.graph_safe() and not self.cache.state
+        # Decode steps are captured into HIP graphs when every part says its launches can be recorded (parts
+        # that loop on the host over sequences cannot).  A part with fixed-size state that says so indexes its
+        # state with ctx.slots on the device; the padded rows of a captured step use the cache's spare slot.
+        safe = model.graph_safe()
         self.use_graphs = safe if use_graphs is None else (use_graphs and safe)
         self._graphs = {}
         self._max_graphs = max_graphs
@@ -189,6 +203,10 @@ class Engine:
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
+
+    @property
+    def page_size(self) -> int:
+        return self.cache.page_size
 
     # ------------------------------------------------------------------ the step
     def step(self, slots: Sequence[int], new_tokens: Sequence[Sequence[int]], want: Want = "last") -> torch.Tensor:
@@ -275,14 +293,18 @@ class Engine:
             self._graphs[key] = self._graphs.pop(key)          # most recently used last
         g.fill(self, slots, tokens, start)
         if g.graph is None:
+            # The first step of a bucket runs eagerly (which also warms up whatever the capture must not do for
+            # the first time) and is then recorded without being run again: a part with state of its own would
+            # otherwise advance that state twice.
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                self.model.forward(g.ctx, self.cache, g.block_tables)      # runs this very step once, eagerly
+                first = self.model.forward(g.ctx, self.cache, g.block_tables)
             torch.cuda.current_stream().wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 g.logits = self.model.forward(g.ctx, self.cache, g.block_tables)
             g.graph = graph
+            return first[:B].clone()
         g.graph.replay()
         return g.logits[:B].clone()                          # the graph's own buffer is overwritten by its next replay

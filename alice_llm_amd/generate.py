@@ -2,9 +2,10 @@
 
 Option names and meanings follow the reference's generate examples where it has them
 (--model, --max-tokens default 256, --temperature, --top-k: examples/elyza_gguf.rs:81-117 and
-examples/generate_gpu.rs:31-40; temperature 0 is greedy, generate_gpu.rs:122; --logits-dump N writes
-the top-5 logits of the first N generated positions as JSON lines to stderr,
-examples/elyza_gguf.rs:31-76).  There is no tokenizer here: prompts are token ids, and so is the
+examples/generate_gpu.rs:31-40; temperature 0 is greedy, generate_gpu.rs:122; --logits-dump N writes,
+for every request, the top-5 logits of its first N generated positions as JSON lines to stderr while the
+request runs: the logits of the run's own steps and the token its sampler drew from them,
+examples/elyza_gguf.rs:31-76, 200-259).  There is no tokenizer here: prompts are token ids, and so is the
 output.  The closing lines are the reference's (examples/elyza_gguf.rs:277-286).
 """
 from __future__ import annotations
@@ -37,7 +38,10 @@ def main(argv=None) -> int:
     ap.add_argument("--stop-ids", default=None, help="stop token ids '1,107' (default: the configuration's eos)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32", "bf16", "fp32"], default=None)
     ap.add_argument("--max-batch", type=int, default=None, help="most sequences in one batch")
-    ap.add_argument("--logits-dump", type=int, default=0, help="dump top-5 logits of the first N generated positions")
+    ap.add_argument("--logits-dump", type=int, default=0,
+                    help="dump the top-5 logits of each request's first N generated positions (JSON lines on stderr)")
+    ap.add_argument("--ignore-unexpected-tensors", action="store_true",
+                    help="tensors in the folder that the model does not declare are warned about instead of refused")
     args = ap.parse_args(argv)
 
     import alice_llm_amd as alice
@@ -62,14 +66,13 @@ def main(argv=None) -> int:
         if not args.model:
             ap.error("give --model DIR, or --random-weights with --preset/--config")
         print(f"Loading model: {args.model}", flush=True)
-        model = alice.load(args.model, dtype=args.dtype)
+        model = alice.load(args.model, dtype=args.dtype, strict=not args.ignore_unexpected_tensors)
 
     stop = _ids(args.stop_ids) if args.stop_ids is not None else None
-    if args.logits_dump > 0:
-        _dump_logits(model, prompts, args.logits_dump)
     results = model.generate(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
                              top_k=args.top_k, top_p=args.top_p, seed=args.seed, stop_token_ids=stop,
-                             max_batch=args.max_batch)
+                             max_batch=args.max_batch,
+                             observer=_logits_dumper(args.logits_dump) if args.logits_dump > 0 else None)
     for i, r in enumerate(results):
         print(f"[{i}] " + ",".join(str(t) for t in r.tokens) + f"  ({r.finish_reason})")
     print("---")
@@ -88,20 +91,25 @@ def main(argv=None) -> int:
     return 0
 
 
-def _dump_logits(model, prompts, n: int) -> None:
-    """Greedy replay of the first prompt, one JSON line per position: the prompt's end, then n - 1 decoded tokens."""
+def _logits_dumper(n: int):
+    """An observer of the generation loop: for each request's first n generated positions one JSON line with
+    the request, the position the logits belong to, the token drawn there and the five largest logits."""
     import torch
-    eng = model.engine(max_tokens=-(-(len(prompts[0]) + n) // 64) * 64, max_seqs=1)
-    slot = eng.open(1)
-    feed = list(prompts[0])
-    for i in range(n):
-        logits = eng.step(slot, [feed], "last")[0]
-        top = torch.topk(logits, min(5, logits.numel()))
-        print(json.dumps({"position": eng.length(slot[0]) - 1,
-                          "top5": [[int(j), float(v)] for v, j in zip(top.values.tolist(), top.indices.tolist())]}),
-              file=sys.stderr, flush=True)
-        feed = [int(top.indices[0])]
-    eng.close(slot)
+    seen = {}
+
+    def observe(requests, positions, logits, tokens) -> None:
+        rows = [i for i, r in enumerate(requests) if seen.get(r, 0) < n]
+        if not rows:
+            return
+        top = torch.topk(logits[rows], min(5, logits.shape[1]), dim=-1)
+        values, indices = top.values.tolist(), top.indices.tolist()
+        for j, i in enumerate(rows):
+            r = requests[i]
+            seen[r] = seen.get(r, 0) + 1
+            print(json.dumps({"request": r, "position": positions[i], "token": int(tokens[i]),
+                              "top5": [[int(t), float(v)] for t, v in zip(indices[j], values[j])]}),
+                  file=sys.stderr, flush=True)
+    return observe
 
 
 if __name__ == "__main__":

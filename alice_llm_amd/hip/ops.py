@@ -403,6 +403,8 @@ def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
 
 
 KV_ROW, KV_FRAGMENT = 0, 1
+KV_FRAGMENT_PAGE = 64            # positions per page that the fragment layout of keys and values is written for
+ATTENTION_MAX_HEAD_DIM = 256     # the largest head size any attention kernel here takes
 
 
 def attention_mfma_supported(head_dim: int) -> bool:

@@ -27,6 +27,10 @@ class Attention(Part):
                  window: Optional[int] = None, position: Optional[str] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
+        if not 1 <= head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
+            # refused when the model is put together, not at its first step
+            raise ValueError(f"attention: head_dim {head_dim} is outside 1..{ops.ATTENTION_MAX_HEAD_DIM}, the range "
+                             f"of the attention kernels")
         self.precision = precision
         self.H, self.nH, self.nKV, self.d = hidden_size, num_heads, num_kv_heads, head_dim
         self.scale = float(scale)
@@ -52,7 +56,9 @@ class Attention(Part):
                 "o_proj.weight": ParamSpec((self.H, self.q_dim))}
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window))
+        # the fragment layout of the matrix-core kernels is written for pages of 64 positions
+        page = ops.KV_FRAGMENT_PAGE if self.kv_layout == ops.KV_FRAGMENT else None
+        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window, page_size=page))
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         if name == "o_proj.weight":

@@ -98,16 +98,26 @@ class Part:
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values that grow with the sequence: rows of num_kv_heads x head_dim per position;
-    `window` keys back from the newest are ever read (None: all of them)."""
+    """Keys and values that grow with the sequence: per position, num_kv_heads rows of head_dim keys and of
+    value_head_dim values (None: the same as the keys); `window` keys back from the newest are ever read
+    (None: all of them).  `page_size`: the number of positions per page that the mixer's kernels are written
+    for (None: any); a cache built with another page size refuses the mixer when the model is put together."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_head_dim: Optional[int] = None
+    page_size: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_head_dim is None else self.value_head_dim
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """State of fixed size per sequence, zero when the sequence starts."""
+    """One tensor of fixed size per sequence, zero when the sequence starts.  A mixer may declare several
+    (a convolution tail and a recurrent matrix, say); it finds each under its name in LayerCache.state."""
+    name: str
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
 
@@ -115,7 +125,17 @@ class StateNeed:
 @dataclass(frozen=True)
 class CacheNeed:
     kv: Optional[KVNeed] = None
-    state: Optional[StateNeed] = None
+    state: Tuple[StateNeed, ...] = ()
+
+    def __post_init__(self):
+        st = self.state
+        if isinstance(st, StateNeed):
+            st = (st,)
+        st = tuple(st or ())
+        names = [s.name for s in st]
+        if len(set(names)) != len(names):
+            raise ValueError(f"state tensors of one part need distinct names, found {names}")
+        object.__setattr__(self, "state", st)
 
 
 # --------------------------------------------------------------------------- registries

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import json
 import os
+import warnings
 from typing import Callable, Dict, Iterable, Iterator, List, Optional, Tuple
 
 import torch
@@ -40,7 +41,14 @@ _FLOAT_OK = (torch.float32, torch.bfloat16)
 _INT_OK = (torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8)
 
 
-def check_tensors(where: str, specs: Dict[str, ParamSpec], found: Dict[str, Tuple[torch.dtype, Tuple[int, ...]]]) -> None:
+class UnexpectedTensorsWarning(UserWarning):
+    """A model folder holds tensors that the model does not declare; they were left unread (strict=False)."""
+
+
+def check_tensors(where: str, specs: Dict[str, ParamSpec], found: Dict[str, Tuple[torch.dtype, Tuple[int, ...]]],
+                  strict: bool = True) -> List[str]:
+    """Raises one WeightError that lists every problem.  Tensors that the model does not declare are a problem
+    when `strict`; otherwise they are returned (and listed in the error only if there is another problem)."""
     missing = [n for n in specs if n not in found]
     unexpected = sorted(n for n in found if n not in specs)
     wrong = []
@@ -54,8 +62,9 @@ def check_tensors(where: str, specs: Dict[str, ParamSpec], found: Dict[str, Tupl
             wrong.append(f"{n}: expected an integer table, found {dt}")
         elif not spec.integer and dt not in _FLOAT_OK:
             wrong.append(f"{n}: dtype {dt} has no kernel (float32 and bfloat16 only)")
-    if missing or unexpected or wrong:
+    if missing or wrong or (unexpected and strict):
         raise WeightError(where, missing, unexpected, wrong)
+    return unexpected
 
 
 def _place(model, name: str, spec: ParamSpec, t: torch.Tensor) -> None:
@@ -64,14 +73,21 @@ def _place(model, name: str, spec: ParamSpec, t: torch.Tensor) -> None:
     model.assign(name, t.to(model.device, non_blocking=False))
 
 
-def load_weights(model, folder: str) -> None:
+def load_weights(model, folder: str, strict: bool = True) -> List[str]:
+    """Fill the model from a folder.  strict: tensors that the model does not declare are an error (listed with
+    the missing and the misshapen ones); otherwise they stay unread, are named in one UnexpectedTensorsWarning
+    and returned."""
     src = TensorSource(folder)
     try:
         specs = model.param_specs()
-        check_tensors(folder, specs, {k: src.info(k) for k in src.keys()})
+        unexpected = check_tensors(folder, specs, {k: src.info(k) for k in src.keys()}, strict)
+        if unexpected:
+            warnings.warn(f"{folder}: {len(unexpected)} tensors that the model does not declare were left unread: "
+                          + ", ".join(unexpected), UnexpectedTensorsWarning, stacklevel=2)
         for name, spec in specs.items():
             _place(model, name, spec, src.tensor(name))
         model.finalize()
+        return unexpected
     finally:
         src.close()
 

@@ -58,9 +58,11 @@ def model_folder(name: str, stored: str = "bfloat16", hot: float = 1.0) -> str:
     return folder
 
 
-def plain_model(folder: str):
+def plain_model(folder: str, dense: bool = False):
+    """dense: attention as one masked matrix product per head instead of key by key (the two forms are tested
+    against each other); what sequences of thousands of tokens need."""
     from plain.gemma2_plain import PlainGemma2
-    return PlainGemma2.from_folder(folder)
+    return PlainGemma2.from_folder(folder, dense=dense)
 
 
 def random_tokens(vocab: int, n: int, seed: int):

@@ -103,22 +103,22 @@ def attention_core(q, k, v, scale, cap, window):
 
 
 def attention_dense(q, k, v, scale, cap, window):
-    """The same attention through one masked matrix product per head (second form)."""
+    """The same attention through one masked matrix product per head (second form; the one long sequences use)."""
     T, nH, d = q.shape
     nKV = k.shape[1]
     g = nH // nKV
-    kk = k.repeat_interleave(g, dim=1)
-    vv = v.repeat_interleave(g, dim=1)
-    s = torch.einsum("thd,uhd->htu", q, kk) * scale
-    s = softcap(s, cap)
     i = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]
     allowed = j <= i
     if window is not None:
         allowed = allowed & (j >= i + 1 - window)
-    s = s.masked_fill(~allowed[None], float("-inf"))
-    p = torch.softmax(s, dim=-1)
-    return torch.einsum("htu,uhd->thd", p, vv)
+    out = torch.empty(T, nH, d, dtype=q.dtype)
+    for h in range(nH):
+        s = (q[:, h, :] @ k[:, h // g, :].T) * scale
+        s = softcap(s, cap)
+        s = s.masked_fill(~allowed, float("-inf"))
+        out[:, h, :] = torch.softmax(s, dim=-1) @ v[:, h // g, :]
+    return out
 
 
 def geglu(x, w_gate, w_up, w_down):
@@ -131,9 +131,10 @@ def geglu(x, w_gate, w_up, w_down):
 class PlainGemma2:
     """Whole-sequence forward from a model folder's raw config.json and tensors."""
 
-    def __init__(self, config: dict, tensors: dict, dtype=DT):
+    def __init__(self, config: dict, tensors: dict, dtype=DT, dense: bool = False):
         c = config
         self.dtype = dtype
+        self.attention = attention_dense if dense else attention_core
         self.V = c["vocab_size"]
         self.H = c["hidden_size"]
         self.L = c["num_hidden_layers"]
@@ -150,7 +151,7 @@ class PlainGemma2:
         self.t = {k: v.to(dtype) for k, v in tensors.items()}
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=DT):
+    def from_folder(cls, folder: str, dtype=DT, dense: bool = False):
         from safetensors import safe_open
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
@@ -158,7 +159,7 @@ class PlainGemma2:
         with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
             for k in f.keys():
                 tensors[k] = f.get_tensor(k)
-        return cls(config, tensors, dtype)
+        return cls(config, tensors, dtype, dense)
 
     def layer_window(self, i: int):
         """Even layers slide, odd layers see everything.  llama3.rs:4634-4641."""
@@ -187,7 +188,7 @@ class PlainGemma2:
         v = (n @ t[p + "self_attn.v_proj.weight"].T).view(T, self.nKV, self.d)
         q = rope_half_split(q, positions, self.theta)
         k = rope_half_split(k, positions, self.theta)
-        o = attention_core(q, k, v, self.scale, self.cap_a, self.layer_window(i))
+        o = self.attention(q, k, v, self.scale, self.cap_a, self.layer_window(i))
         a = o.reshape(T, self.nH * self.d) @ t[p + "self_attn.o_proj.weight"].T
         if taps is not None:
             taps[f"layer{i}.attn_out"] = a

@@ -103,20 +103,42 @@ def test_random_traffic_loses_nothing():
 
 
 def test_state_region_is_zeroed_on_open():
-    c = Cache([CacheNeed(state=StateNeed((3, 2)))], max_tokens=128, dtype=torch.float32, device="cpu", max_seqs=2)
-    assert c.state[0].shape == (2, 3, 2) and not c.groups
-    s = c.open(); c.state[0][s] += 5; c.close(s)
+    # two tensors of different shape and dtype for one run of the schedule, a row per slot and a spare row
+    need = CacheNeed(state=(StateNeed("tail", (3, 2)), StateNeed("matrix", (4,), torch.float64)))
+    c = Cache([need, None, CacheNeed(state=StateNeed("s", (1,)))], max_tokens=128, dtype=torch.float32, device="cpu", max_seqs=2)
+    assert sorted(c.state) == [0, 2] and not c.groups and c.spare_slot == 2
+    assert c.state[0]["tail"].shape == (3, 3, 2) and c.state[0]["matrix"].dtype == torch.float64
+    s = c.open(); c.state[0]["tail"][s] += 5; c.state[0]["matrix"][s] -= 1; c.close(s)
     s2 = c.open()
-    assert s2 == s and float(c.state[0][s2].abs().sum()) == 0.0
+    assert s2 == s and all(float(t[s2].abs().sum()) == 0.0 for t in c.state[0].values())
+    view = c.view(0, [])
+    assert set(view.state) == {"tail", "matrix"} and c.view(1, []).state == {}
+    with pytest.raises(ValueError, match="distinct names"):
+        CacheNeed(state=(StateNeed("a", (1,)), StateNeed("a", (2,))))
+
+
+def test_page_size_is_the_caches_and_parts_can_insist_on_theirs():
+    c = Cache(needs(), max_tokens=100, dtype=torch.float32, device="cpu", allocate=False, page_size=16)
+    assert c.page_size == 16 and c.max_tokens == 112
+    s = c.open(); c.reserve([s], [40]); c.commit([s], [40])
+    assert len(c.groups[1].table(s)) == 3
+    with pytest.raises(CacheError, match="pages of 64"):
+        Cache([CacheNeed(kv=KVNeed(1, 16, None, page_size=64))], max_tokens=100, dtype=torch.float32, device="cpu",
+              allocate=False, page_size=16)
+    # keys and values of different head sizes get storage of their own shapes
+    c = Cache([CacheNeed(kv=KVNeed(2, 16, None, value_head_dim=8))], max_tokens=64, dtype=torch.float32, device="cpu")
+    assert c.groups[0].k.shape == (1, 2, 2, 64, 16) and c.groups[0].v.shape == (1, 2, 2, 64, 8)
 
 
 # ------------------------------------------------------------------ the loop
 class FakeEngine:
     """Scripted logits: token = (last token fed + 1) mod V for every sequence; records slot traffic."""
 
-    def __init__(self, V=16, max_tokens=64 * 8, n_slots=4):
+    def __init__(self, V=16, max_tokens=64 * 8, n_slots=4, max_positions=None, page_size=64):
         self.V = V
-        self.cache = make(max_tokens=max_tokens, max_seqs=n_slots)
+        if max_positions is not None:
+            self.max_positions = max_positions
+        self.cache = make(max_tokens=max_tokens, max_seqs=n_slots, page_size=page_size)
         self.opened, self.closed, self.steps = [], [], []
 
     def open(self, n):
@@ -143,10 +165,46 @@ def argmax_sampler(logits, requests, draws):
 
 
 def test_plan_batches():
-    assert plan_batches([5, 12, 17, 100], [8] * 4, max_batch=2, capacity_tokens=256, max_slots=4) == [[0, 1], [2, 3]]
-    assert plan_batches([60, 60, 60], [10] * 3, max_batch=None, capacity_tokens=256, max_slots=8) == [[0, 1], [2]]
+    assert plan_batches([5, 12, 17, 100], [8] * 4, max_batch=2, capacity_tokens=256, max_slots=4, page=64) == [[0, 1], [2, 3]]
+    assert plan_batches([60, 60, 60], [10] * 3, max_batch=None, capacity_tokens=256, max_slots=8, page=64) == [[0, 1], [2]]
+    # the page size is the cache's: with pages of 16 the same three requests (69 tokens -> 80 each) fit together
+    assert plan_batches([60, 60, 60], [10] * 3, max_batch=None, capacity_tokens=256, max_slots=8, page=16) == [[0, 1, 2]]
+    # the last token drawn is never fed back: 60 + 5 - 1 = 64 tokens are one page
+    assert plan_batches([60, 60], [5, 5], max_batch=None, capacity_tokens=128, max_slots=8, page=64) == [[0, 1]]
     with pytest.raises(ValueError, match="request 1"):
-        plan_batches([5, 300], [8, 8], max_batch=4, capacity_tokens=256, max_slots=4)
+        plan_batches([5, 300], [8, 8], max_batch=4, capacity_tokens=256, max_slots=4, page=64)
+
+
+def test_requests_that_would_outgrow_the_positions():
+    from alice_llm_amd.engine.generate import limit_caps
+    assert limit_caps([5, 10, 3], [100, 2, 0], 12) == [8, 2, 0]       # 5 + 8 - 1 = 12 positions; small caps untouched
+    with pytest.raises(ValueError, match="request 1.*13 tokens"):
+        limit_caps([5, 13], [1, 1], 12)
+    # in the loop: the long request ends with "length" at the last position, its batch mates are untouched, and
+    # no step ever asks the engine for a position beyond the limit
+    eng = FakeEngine(max_positions=12)
+    res = Generator(eng, stop_token_ids=[], sampler=argmax_sampler).run([[1, 2, 3, 4, 5], [7], [9, 10]], [100, 3, 4])
+    assert [len(r.tokens) for r in res] == [8, 3, 4] and [r.finish_reason for r in res] == ["length"] * 3
+    assert res[0].tokens == [6, 7, 8, 9, 10, 11, 12, 13]
+    assert max(sum(n for sl, ns in eng.steps for s, n in zip(sl, ns) if s == slot) for slot in range(3)) == 12
+    assert eng.cache.slots.n_free() == 4
+    # a prompt that is too long is refused before any slot is taken or any step runs
+    eng = FakeEngine(max_positions=12)
+    with pytest.raises(ValueError, match="request 2"):
+        Generator(eng, sampler=argmax_sampler).run([[1], [2], list(range(13))], [2, 2, 2])
+    assert eng.opened == [] and eng.steps == []
+
+
+def test_loop_observer_sees_the_runs_own_steps():
+    seen = []
+    def observer(requests, positions, logits, tokens):
+        seen.append((list(requests), list(positions), logits.argmax(-1).tolist(), list(tokens)))
+    gen = Generator(FakeEngine(), stop_token_ids=[9], sampler=argmax_sampler, observer=observer)
+    res = gen.run([[1, 2, 3], [7]], [3, 5])
+    assert [r.tokens for r in res] == [[4, 5, 6], [8]]
+    # the first step's logits belong to the prompts' last positions; the stop token is seen though not kept
+    assert seen[0] == ([0, 1], [2, 0], [4, 8], [4, 8]) and seen[1] == ([0, 1], [3, 1], [5, 9], [5, 9])
+    assert seen[2] == ([0], [4], [6], [6]) and len(seen) == 3
 
 
 def test_loop_stop_tokens_caps_and_slot_reuse():

@@ -45,6 +45,8 @@ def test_config_defaults_and_nulls():
     ({"num_key_value_heads": 3}, "divide"), ({"head_dim": 15}, "even"), ({"sliding_window": 0}, "sliding_window"),
     ({"final_logit_softcapping": -1.0}, "final_logit_softcapping"), ({"hidden_activation": "silu"}, "gelu_pytorch_tanh"),
     ({"architectures": ["LlamaForCausalLM"]}, "registered"), ({"num_hidden_layers": True}, "integer"),
+    # keys that would change the arithmetic and that nothing implements are refused, not dropped
+    ({"attention_bias": True}, "attention_bias"), ({"rope_scaling": {"type": "linear", "factor": 2.0}}, "rope_scaling"),
 ])
 def test_config_errors_name_the_key(change, word):
     d = dict(TINY_A)
@@ -117,6 +119,25 @@ def test_weight_error_lists_everything_at_once():
         assert word in msg
     untied = _specs_without_device(alice.config_from_dict(dict(TINY_A, tie_word_embeddings=False)))
     assert untied["lm_head.weight"].shape == (256, 64)
+    # not strict: tensors that the model does not declare are handed back instead of refused, alone ...
+    ok = {n: (torch.bfloat16, s.shape) for n, s in specs.items()}
+    ok["rotary.inv_freq"] = (torch.float32, (8,))
+    assert check_tensors("folder", specs, ok, strict=False) == ["rotary.inv_freq"]
+    with pytest.raises(WeightError, match="unexpected \\(1\\): rotary.inv_freq"):
+        check_tensors("folder", specs, ok)
+    # ... and still listed beside any other problem
+    del ok["model.norm.weight"]
+    with pytest.raises(WeightError) as e:
+        check_tensors("folder", specs, ok, strict=False)
+    assert e.value.unexpected == ["rotary.inv_freq"] and e.value.missing == ["model.norm.weight"]
+
+
+def test_a_head_size_beyond_the_kernels_is_refused_when_the_model_is_put_together():
+    from alice_llm_amd.config import ConfigError
+    cfg = alice.config_from_dict(dict(TINY_A, head_dim=272, query_pre_attn_scalar=272))
+    with pytest.raises(ValueError, match="head_dim 272"):
+        _specs_without_device(cfg)
+    assert alice.config_from_dict(dict(TINY_A, attention_bias=False, rope_scaling=None)).head_dim == 16
 
 
 def test_random_weights_folder():

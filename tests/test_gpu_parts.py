@@ -169,19 +169,20 @@ class ToyDecayMixer(Part):
         self.w[name] = t.float()
 
     def cache_need(self):
-        return CacheNeed(state=StateNeed((self.S,), torch.float32))
+        return CacheNeed(state=StateNeed("s", (self.S,), torch.float32))
 
     def forward(self, x, ctx, cache):
         u = x.float() @ self.w["in.weight"].T
         out = torch.empty_like(u)
         row = 0
+        state = cache.state["s"]
         for slot, n in zip(ctx.slot_ids, ctx.new_lens):
-            s = cache.state[slot]
+            s = state[slot]
             for i in range(n):
                 s = self.decay * s + u[row]
                 out[row] = s
                 row += 1
-            cache.state[slot] = s
+            state[slot] = s
         return (out @ self.w["out.weight"].T).contiguous()
 
 
@@ -325,6 +326,144 @@ def test_toy_architecture_against_its_plain_replica():
     got = torch.cat([eng.step(s, [toks[:9]], "all")] + [eng.step(s, [[t]], "last") for t in toks[9:]])
     ref = toy_plain(model, toks)
     assert (got.double().cpu() - ref).abs().max() < 2e-5 * max(1.0, float(ref.abs().max()))
+
+
+# ------------------------------------------------------------------ a toy with two state tensors, in captured steps
+class ToyTailScanMixer(Part):
+    """A mixer with two state tensors per sequence, of different shapes: the last two inputs (a convolution's
+    tail) and a running sum.  c_t = u_t + 0.5 u_(t-1) + 0.25 u_(t-2) with u = x W_in, s_t = decay * s_(t-1) + c_t,
+    output s_t W_out.  Single-token steps index the state with ctx.slots on the device and launch the same
+    kernels whatever the batch holds, so the mixer declares graph_safe and its decode steps are captured into
+    HIP graphs; prompts loop on the host."""
+    graph_safe = True
+
+    def __init__(self, precision, positions, *, hidden_size, state_size, decay):
+        self.H, self.S, self.decay = hidden_size, state_size, decay
+        self.w = {}
+
+    def param_specs(self):
+        return {"in.weight": ParamSpec((self.S, self.H), 0.1), "out.weight": ParamSpec((self.H, self.S), 0.1)}
+
+    def assign(self, name, t):
+        self.w[name] = t.float()
+
+    def cache_need(self):
+        return CacheNeed(state=(StateNeed("tail", (2, self.S)), StateNeed("sum", (self.S,))))
+
+    def forward(self, x, ctx, cache):
+        u = x.float() @ self.w["in.weight"].T
+        tail, acc = cache.state["tail"], cache.state["sum"]
+        if ctx.is_decode:
+            idx = ctx.slots.long()                             # device data: the same launches for any batch
+            t = tail.index_select(0, idx)                      # [B, 2, S]: u_(t-2), u_(t-1)
+            s = self.decay * acc.index_select(0, idx) + u + 0.5 * t[:, 1] + 0.25 * t[:, 0]
+            acc.index_copy_(0, idx, s)
+            tail.index_copy_(0, idx, torch.stack([t[:, 1], u], dim=1))
+            out = s
+        else:
+            assert not ctx.captured
+            out = torch.empty_like(u)
+            row = 0
+            for slot, n in zip(ctx.slot_ids, ctx.new_lens):
+                t2, t1, s = tail[slot, 0].clone(), tail[slot, 1].clone(), acc[slot].clone()
+                for _ in range(n):
+                    s = self.decay * s + u[row] + 0.5 * t1 + 0.25 * t2
+                    out[row] = s
+                    t2, t1 = t1, u[row]
+                    row += 1
+                tail[slot, 0], tail[slot, 1], acc[slot] = t2, t1, s
+        return (out @ self.w["out.weight"].T).contiguous()
+
+
+class ToyGraphMLP(ToyMLP):
+    graph_safe = True
+
+
+class ToyScanConfig(ToyConfig):
+    def plan(self):
+        H, V = self.d["width"], self.d["vocab"]
+        norm = lambda name: PartSpec("rmsnorm", {"dim": H, "eps": 1e-5, "weight_offset": 0.0}, name)
+        scan = lambda: PartSpec("toy_tail_scan", {"hidden_size": H, "state_size": self.d["state"], "decay": 0.75}, "mix")
+        att = PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "scale": 0.25,
+                                     "window": 7, "position": "rope"}, "attn")
+        layers = [LayerPlan(block="prenorm", mixer=m, feed_forward=PartSpec("toy_graph_mlp", {"hidden_size": H}, "ff"),
+                            norms={"pre_mixer": norm("n1"), "pre_ff": norm("n2")}, prefix=f"blocks.{i}.")
+                  for i, m in enumerate([scan(), att, scan()])]
+        return ModelPlan(vocab_size=V, hidden_size=H, max_positions=256,
+                         embedding=PartSpec("embedding", {"vocab_size": V, "dim": H, "scale": 1.0}, "emb"),
+                         positions={"rope": PartSpec("rope", {"dim": 16, "theta": 100.0, "max_positions": 256})},
+                         layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(3)),
+                         final_norm=norm("final"), head=PartSpec("lm_head", {"vocab_size": V, "dim": H, "tied_to": "emb"}, "head"))
+
+
+def toy_scan_plain(model, tokens):
+    lm = model.lm
+    E = lm.embedding.table.weight.double().cpu()
+    x = E[torch.tensor(tokens)]
+    T = len(tokens)
+    rms = lambda v, n: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + n.eps) * (n.weight_offset + n.weight.double().cpu())
+    for layer in lm.layers:
+        h = rms(x, layer.norms["pre_mixer"])
+        m = layer.mixer
+        if isinstance(m, ToyTailScanMixer):
+            u = h @ m.w["in.weight"].double().cpu().T
+            s, outs = torch.zeros(m.S, dtype=D), []
+            for i in range(T):
+                s = 0.75 * s + u[i] + (0.5 * u[i - 1] if i >= 1 else 0) + (0.25 * u[i - 2] if i >= 2 else 0)
+                outs.append(s)
+            a = torch.stack(outs) @ m.w["out.weight"].double().cpu().T
+        else:
+            W = m.qkv.weight.double().cpu()
+            if m.pair_order:
+                W = torch.empty_like(W).index_copy_(0, m.position.projection_row_order(2, 1, 16), W)
+            pos = torch.arange(T)
+            q, k, v = (h @ W[:32].T).view(T, 2, 16), (h @ W[32:48].T).view(T, 1, 16), (h @ W[48:64].T).view(T, 1, 16)
+            o = P.attention_core(P.rope_half_split(q, pos, 100.0), P.rope_half_split(k, pos, 100.0), v, 0.25, None, 7)
+            a = o.reshape(T, 32) @ m.o.weight.double().cpu().T
+        x = x + a
+        x = x + torch.relu(rms(x, layer.norms["pre_ff"]) @ layer.feed_forward.w.double().cpu().T)
+    return rms(x, lm.final_norm) @ E.T
+
+
+def test_toy_mixer_with_two_state_tensors_runs_in_captured_steps():
+    MIXERS.register("toy_tail_scan", ToyTailScanMixer)
+    FEED_FORWARDS.register("toy_graph_mlp", ToyGraphMLP)
+    alice.register_architecture("ToyScanForCausalLM", ToyScanConfig)
+    raw = {"architectures": ["ToyScanForCausalLM"], "width": 48, "vocab": 83, "state": 20}
+    model = alice.Model.random(raw, seed=6, dtype="float32", stored_dtype=torch.float32)
+    graph = model.engine(max_tokens=64 * 6, max_seqs=5)
+    eager = model.engine(max_tokens=64 * 6, max_seqs=5, use_graphs=False)
+    assert graph.use_graphs and not eager.use_graphs            # state does not turn captured steps off
+    assert sorted(graph.cache.state) == [0, 2] and set(graph.cache.state[0]) == {"tail", "sum"}
+    assert graph.cache.state[0]["tail"].shape == (5 + 1, 2, 20)   # a row per slot and the spare one
+    g = torch.Generator().manual_seed(9)
+    seqs = [torch.randint(0, 83, (n,), generator=g).tolist() for n in (30, 12, 21)]
+    prompt = [4, 1, 9]
+    refs = [toy_scan_plain(model, t) for t in seqs]
+    for again in range(2):                                       # a second batch on the same slots: state starts at zero
+        got = {}
+        for eng in (graph, eager):
+            slots = eng.open(3)
+            first = eng.step(slots, [s[:n] for s, n in zip(seqs, prompt)], "all")
+            outs, o = {}, 0
+            for i, n in enumerate(prompt):
+                outs[i] = [first[o:o + n]]
+                o += n
+            live, step = [0, 1, 2], 0
+            while live:                                           # three rows in a captured step of four: one padded row
+                lg = eng.step([slots[i] for i in live], [[seqs[i][prompt[i] + step]] for i in live], "last")
+                for row, i in enumerate(live):
+                    outs[i].append(lg[row:row + 1].clone())
+                step += 1
+                done = [i for i in live if prompt[i] + step >= len(seqs[i])]
+                eng.close([slots[i] for i in done])
+                live = [i for i in live if i not in done]
+            got[eng] = [torch.cat(outs[i]) for i in range(3)]
+            eng.cache.check_consistent()
+        for i in range(3):
+            assert (got[graph][i].double().cpu() - refs[i]).abs().max() < 2e-5 * max(1.0, float(refs[i].abs().max())), (again, i)
+            assert (got[graph][i] - got[eager][i]).abs().max() < 1e-5
+    assert len(graph._graphs) >= 3                               # batches of 3 (a bucket of 4), 2 and 1
 
 
 # ------------------------------------------------------------------ a second toy: routing and another position encoding

@@ -152,29 +152,113 @@ def test_gelu_is_the_tanh_form():
 
 
 # ------------------------------------------------------------------ whole model
+def small_plain(L, W, H=32, seed=0, **over):
+    """A plain model of L layers from a configuration and random tensors made here."""
+    cfg = dict(vocab_size=50, hidden_size=H, num_hidden_layers=L, num_attention_heads=2, num_key_value_heads=1, head_dim=8,
+               intermediate_size=48, rope_theta=100.0, rms_norm_eps=1e-6, sliding_window=W, attn_logit_softcapping=50.0,
+               final_logit_softcapping=30.0, query_pre_attn_scalar=8)
+    cfg.update(over)
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *shape, std=0.3: torch.randn(*shape, generator=g, dtype=D) * std
+    t = {"model.embed_tokens.weight": r(cfg["vocab_size"], H), "model.norm.weight": r(H, std=0.1)}
+    for i in range(L):
+        p = f"model.layers.{i}."
+        t[p + "self_attn.q_proj.weight"], t[p + "self_attn.o_proj.weight"] = r(16, H), r(H, 16)
+        t[p + "self_attn.k_proj.weight"], t[p + "self_attn.v_proj.weight"] = r(8, H), r(8, H)
+        t[p + "mlp.gate_proj.weight"], t[p + "mlp.up_proj.weight"], t[p + "mlp.down_proj.weight"] = r(48, H), r(48, H), r(H, 48)
+        for n in ("input", "post_attention", "pre_feedforward", "post_feedforward"):
+            t[p + n + "_layernorm.weight"] = r(H, std=0.1)
+    return P.PlainGemma2(cfg, t)
+
+
+def test_which_layers_slide():
+    """Layer 0 slides and layer 1 is global (llama3.rs:4634-4641).  With one layer, nothing before the window can
+    reach a position; with two, it does, and only through layer 1.  The mistake this catches: the kinds swapped
+    (odd layers sliding), or every layer of one kind."""
+    W, T, p = 4, 14, 13
+    toks = random_tokens(50, T, 1)
+    far = list(toks); far[p - W] = (toks[p - W] + 1) % 50          # the newest token outside position p's window
+    edge = list(toks); edge[p + 1 - W] = (toks[p + 1 - W] + 1) % 50  # the oldest inside it
+    one = small_plain(1, W)
+    assert torch.equal(one.forward(far)[p], one.forward(toks)[p])        # layer 0 slides: bit-equal
+    assert (one.forward(edge)[p] - one.forward(toks)[p]).abs().max() > 1e-6
+    two = small_plain(2, W)
+    assert (two.forward(far)[p] - two.forward(toks)[p]).abs().max() > 1e-6      # layer 1 sees everything
+    # only through layer 1: the far token reaches p in layer 1 directly, so layer 0's output at p is still bit-equal
+    taps_a, taps_b = {}, {}
+    two.forward(far, taps_a); two.forward(toks, taps_b)
+    assert torch.equal(taps_a["layer0.out"][p], taps_b["layer0.out"][p])
+    assert not torch.equal(taps_a["layer1.attn_out"][p], taps_b["layer1.attn_out"][p])
+    # with three layers the third slides again: a token two windows back reaches p only through layer 1
+    three = small_plain(3, W)
+    assert [three.layer_window(i) for i in range(3)] == [W, None, W]
+
+
+def test_scale_comes_before_the_cap():
+    """score * scale, then cap * tanh(. / cap) (llama3.rs:5622-5642).  With cap 0.01 and scale 100 the capped scores
+    lie within +-0.01 whatever the scale, so the softmax is nearly uniform; in the other order (cap, then scale)
+    they spread over +-1 and it is not."""
+    q, k, v = _qkv(10, 2, 1, 8, 8)
+    for form in (P.attention_core, P.attention_dense):
+        out = form(q, k, v, 100.0, 0.01, None)
+        uniform = v[:, 0].cumsum(0) / torch.arange(1, 11, dtype=D)[:, None]
+        assert (out[:, 0] - uniform).abs().max() < 0.03 * v.abs().max()
+    raw = torch.einsum("td,ud->tu", q[:, 0], k[:, 0])
+    swapped = (0.01 * torch.tanh(raw / 0.01)) * 100.0                    # the mistake
+    swapped = swapped.masked_fill(torch.arange(10)[None, :] > torch.arange(10)[:, None], float("-inf"))
+    assert (torch.softmax(swapped, -1) @ v[:, 0] - uniform).abs().max() > 4 * 0.03 * v.abs().max()
+
+
+def test_the_head_is_the_embedding_matrix():
+    """One matrix serves the embedding and the head (llama3.rs:12896-12906): doubling row v doubles logit v
+    before the cap and nothing else, for sequences without token v; and changes every logit of a sequence that
+    holds token v, because its input changed.  The mistake this catches: a head with a matrix of its own."""
+    m = small_plain(2, 4)
+    v = 17
+    toks = [t for t in random_tokens(50, 12, 2) if t != v]
+    base = m.forward(toks)
+    m2 = small_plain(2, 4)
+    m2.t["model.embed_tokens.weight"][v] *= 2.0
+    out = m2.forward(toks)
+    others = [i for i in range(50) if i != v]
+    assert torch.equal(out[:, others], base[:, others])
+    precap = lambda z: 30.0 * torch.atanh(z / 30.0)
+    assert torch.allclose(precap(out[:, v]), 2.0 * precap(base[:, v]), atol=1e-9)
+    with_v = toks[:5] + [v] + toks[5:]
+    assert (m2.forward(with_v)[6:, others] - m.forward(with_v)[6:, others]).abs().max() > 1e-6
+
+
+def test_embedding_scale_is_the_square_root_taken_in_f32():
+    """x = E[token] * sqrt(width), the root taken of the width as an f32 (llama3.rs:13697-13703).  For a width of
+    96 that is 9.797959327697754, not the 64-bit root 9.797958971132712; no factor on the way out."""
+    m = small_plain(1, 4, H=96)
+    E = m.t["model.embed_tokens.weight"]
+    assert torch.equal(m.embed([5, 9]), E[[5, 9]] * 9.797959327697754)
+    assert not torch.equal(m.embed([5]), E[[5]] * math.sqrt(96.0))
+    assert torch.equal(small_plain(1, 4, H=64).embed([3]), small_plain(1, 4, H=64).t["model.embed_tokens.weight"][[3]] * 8.0)
+
+
 @pytest.mark.parametrize("name", ["tiny-a", "tiny-b"])
 def test_model_invariants(name):
-    folder = model_folder(name, "float32")
-    m = plain_model(folder)
+    m = plain_model(model_folder(name, "float32"))
     toks = random_tokens(m.V, 20, 3)
     full = m.forward(toks)
-    assert full.shape == (20, m.V) and full.abs().max() < m.cap_f
+    assert full.shape == (20, m.V)
     assert torch.allclose(m.forward(toks[:13]), full[:13], atol=1e-12)           # prefix invariance
-    # tied head: scaling row v of E scales logit v at every position's pre-cap value and token v's input
-    taps = {}
-    m.forward(toks, taps)
-    assert set(taps) >= {"layer0.attn_out", f"layer{m.L - 1}.out"}
+    # the final cap bites where logits are large: the hot variant's logits come near the cap and stay below it,
+    # and without the cap they pass it
+    hot = plain_model(model_folder(name, "float32", hot=12.0))
+    capped = hot.forward(toks)
+    assert 0.4 * hot.cap_f < capped.abs().max() < hot.cap_f
+    hot.cap_f = None
+    assert hot.forward(toks).abs().max() > capped.abs().max() + 0.5
 
 
 def test_model_layer_kinds_and_norm_places():
     folder = model_folder("tiny-b", "float32")
     m = plain_model(folder)
-    assert [m.layer_window(i) for i in range(3)] == [6, None, 6]                # llama3.rs:4636-4641
     toks = random_tokens(m.V, 16, 4)
     base = m.forward(toks)
-    # a far token (position 0) still reaches the end through the global layer only
-    other = list(toks); other[0] = (toks[0] + 1) % m.V
-    assert (m.forward(other)[-1] - base[-1]).abs().max() > 1e-9
     m2 = plain_model(folder); m2.window = 1000
     assert (m2.forward(toks)[-1] - base[-1]).abs().max() > 1e-9                 # the window matters at T=16 > 6
     assert torch.allclose(m2.forward(toks)[:6], base[:6], atol=1e-12)           # and not before it bites
@@ -188,12 +272,6 @@ def test_model_layer_kinds_and_norm_places():
     for i in range(3):
         out = m3.layer(i, out, torch.arange(16))
     assert torch.allclose(out, x, atol=1e-12)
-
-
-def test_embedding_scale():
-    m = plain_model(model_folder("tiny-b", "float32"))
-    e = m.embed([5])
-    assert torch.allclose(e[0], m.t["model.embed_tokens.weight"][5] * float(torch.tensor(96.0).sqrt()), atol=0)
 
 
 # ------------------------------------------------------------------ sampling
