@@ -84,8 +84,102 @@ def test_command_line(tmp_path):
     lines = proc.stdout.splitlines()
     assert f"[0] {','.join(map(str, want[0]))}  (length)" in lines and f"[1] {','.join(map(str, want[1]))}  (length)" in lines
     assert "Tokens: 10 generated, 6 prompt" in lines and any(l.startswith("Speed: ") and "tok/s" in l for l in lines)
-    dumps = [l for l in proc.stderr.splitlines() if l.startswith("{")]
-    assert len(dumps) == 2 and '"position": 3' in dumps[0] and f"[{want[0][0]}," in dumps[0].replace(" ", "").replace("[[", "[")
+    # the dump comes from the run's own steps: both requests, their first two generated positions, the token
+    # the run's sampler drew there, and the plain implementation's five largest logits
+    import json
+    dumps = [json.loads(l) for l in proc.stderr.splitlines() if l.startswith("{")]
+    assert [(d["request"], d["position"]) for d in dumps] == [(0, 3), (1, 1), (0, 4), (1, 2)]
+    for d in dumps:
+        seq = prompts[d["request"]] + want[d["request"]]
+        lg = plain.forward(seq[:d["position"] + 1])[-1]
+        top = torch.topk(lg, 5)
+        assert d["token"] == seq[d["position"] + 1] == d["top5"][0][0]
+        assert [t for t, _ in d["top5"]] == top.indices.tolist()
+        assert max(abs(v - float(w)) for (_, v), w in zip(d["top5"], top.values)) < 2e-5
+
+
+def test_logits_dump_follows_the_sampler_of_the_run():
+    """With a temperature the dumped token is the one that was drawn and kept, which need not be the largest logit."""
+    folder = model_folder("tiny-b", "bfloat16")
+    model = alice.load(folder, dtype="float32")
+    from alice_llm_amd.generate import _logits_dumper
+    import contextlib, io, json
+    err = io.StringIO()
+    with contextlib.redirect_stderr(err):
+        res = model.generate([[3, 4, 5], [9]], max_new_tokens=6, temperature=1.5, seed=3, stop_token_ids=[],
+                             observer=_logits_dumper(4))
+    dumps = [json.loads(l) for l in err.getvalue().splitlines()]
+    assert len(dumps) == 8
+    for r in (0, 1):
+        mine = [d for d in dumps if d["request"] == r]
+        assert [d["token"] for d in mine] == res[r].tokens[:4]
+    assert any(d["token"] != d["top5"][0][0] for d in dumps)
+
+
+def test_a_request_that_reaches_the_last_position_ends_alone():
+    """One request of a batch would outgrow max_position_embeddings (512): it ends with "length" at the last
+    position, its batch mates finish as they would alone, nothing is lost and no slot stays held."""
+    folder = model_folder("tiny-a", "bfloat16")
+    plain = plain_model(folder, dense=True)
+    model = alice.load(folder, dtype="float32")
+    eng = model.engine(seq_lens=[512, 64, 64], max_seqs=3)
+    long_prompt, short = random_tokens(plain.V, 505, 80), random_tokens(plain.V, 9, 81)
+    gen = alice.Generator(eng, stop_token_ids=[])
+    res = gen.run([long_prompt, short, [5]], [40, 12, 3])
+    assert [len(r.tokens) for r in res] == [8, 12, 3] and all(r.finish_reason == "length" for r in res)
+    assert res[0].tokens == plain.greedy(long_prompt, 8) and res[1].tokens == plain.greedy(short, 12)
+    assert eng.cache.slots.n_free() == 3
+    eng.cache.check_consistent()
+    with pytest.raises(ValueError, match="request 1.*513"):
+        gen.run([[1, 2], [3] * 513], [4, 4])
+    assert eng.cache.slots.n_free() == 3
+
+
+def test_sample_and_step_of_the_python_surface():
+    folder = model_folder("tiny-b", "bfloat16")
+    plain = plain_model(folder)
+    model = alice.load(folder, dtype="float32")
+    eng = model.engine(max_tokens=128)
+    toks = random_tokens(plain.V, 12, 90)
+    s = eng.open(1)
+    logits = model.step(eng, s, [toks], "all")                                  # the step function by its other name
+    assert (logits.double().cpu() - plain.forward(toks)).abs().max() < 2e-5
+    other = alice.load(folder, dtype="float32")
+    with pytest.raises(ValueError, match="another model"):
+        other.step(eng, s, [[1]])
+    assert alice.sample(logits).tolist() == logits.argmax(-1).tolist()          # temperature 0: greedy, no u needed
+    assert alice.sample(logits[3]).tolist() == [int(logits[3].argmax())]
+    us = [uniform(5, 0, n) for n in range(12)]
+    got = alice.sample(logits, temperature=0.9, top_k=7, top_p=0.8, u=us).tolist()
+    for row, (g, u) in enumerate(zip(got, us)):
+        want = P.plain_sample(logits[row].double().cpu(), 0.9, 7, 0.8, u)
+        if g != want:                                                           # a draw within rounding of a boundary
+            x = P.plain_top_p(P.plain_top_k(logits[row].double().cpu() / 0.9, 7), 0.8)
+            cdf = torch.cumsum(P.plain_softmax(x), 0)
+            assert abs(float(cdf[min(g, want)]) - u) < 1e-4
+    with pytest.raises(ValueError, match="needs u"):
+        alice.sample(logits, temperature=0.5)
+    with pytest.raises(ValueError, match="one number"):
+        alice.sample(logits, temperature=0.5, u=[0.1, 0.2])
+
+
+def test_unexpected_tensors_are_an_error_or_a_warning(tmp_path):
+    from safetensors.torch import load_file, save_file
+    import shutil, warnings
+    src = model_folder("tiny-a", "bfloat16")
+    folder = str(tmp_path / "extra")
+    shutil.copytree(src, folder)
+    t = load_file(os.path.join(folder, "model.safetensors"))
+    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    save_file(t, os.path.join(folder, "model.safetensors"))
+    with pytest.raises(alice.WeightError, match="unexpected \\(1\\): model.layers.0.self_attn.rotary_emb.inv_freq"):
+        alice.load(folder, dtype="float32")
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        model = alice.load(folder, dtype="float32", strict=False)
+    assert any(issubclass(x.category, alice.UnexpectedTensorsWarning) and "inv_freq" in str(x.message) for x in w)
+    a, b = model.engine(64), alice.load(src, dtype="float32").engine(64)
+    assert torch.equal(a.step(a.open(1), [[1, 2, 3]], "all"), b.step(b.open(1), [[1, 2, 3]], "all"))
 
 
 def test_random_mode_matches_folder():

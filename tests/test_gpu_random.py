@@ -42,7 +42,7 @@ def test_random_configuration_and_schedule(case):
     n_seq = rng.choice([1, 2, 3, 5])
     lens = [rng.choice([1, 17, 64, 65, 130, 200] if big else [1, 2, 15, 16, 17, 33, 64, 65, 100, 130]) for _ in range(n_seq)]
     decode = rng.choice([0, 1, 3, 20])
-    cut = rng.choice([0, 0, 1, 7])
+    cut = rng.choice([0, 0, 1, 7, 64, 70])
     seqs = [random_tokens(plain.V, n + decode, 100 * number + i) for i, n in enumerate(lens)]
     refs = [plain.forward(s) for s in seqs]
     scale = max(1.0, max(float(r.abs().max()) for r in refs))
@@ -54,7 +54,7 @@ def test_random_configuration_and_schedule(case):
             if again:
                 slots = slots[::-1]
             got = [[] for _ in seqs]
-            pieces = [(0, cut), (cut, None)] if cut and all(n > cut for n in lens) else [(0, None)]
+            pieces = [(0, cut), (cut, None)] if cut and all(n > cut for n in lens) else [(0, None)]      # a second piece on a cached prefix
             for a, b in pieces:
                 ends = [n if b is None else b for n in lens]
                 out, o = eng.step(slots, [s[a:e] for s, e in zip(seqs, ends)], "all"), 0

@@ -85,3 +85,35 @@ def test_odd_sizes_whole_and_token_by_token(name):
         eng.close(s)
         assert max_err(whole, ref) < TOL[dtype] * scale, (dtype, max_err(whole, ref))
         assert max_err(torch.cat(cut), ref) < TOL[dtype] * scale, (dtype, max_err(torch.cat(cut), ref))
+
+
+def test_full_2b_shape_bfloat16_against_the_32_bit_path():
+    """The whole Gemma 2 2B shape (26 layers, vocabulary 256,000) with random weights: a prompt of 292 tokens and
+    8 single tokens, the bfloat16 path against the true 32-bit path on the same weights.  The reference checks its
+    quantised forward against an all-f32 one the same way (examples/test_1b.rs:190-227: max and mean difference
+    of the logits).  Bound: the logits (rms about 1, maximum about 8) differ by at most 0.06, and where the
+    two paths choose another token the 32-bit logits of the two are closer than that."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40e9:
+        pytest.skip(f"needs 40 GB of free GPU memory for both models, {free / 1e9:.0f} GB are free")
+    cfg = alice.config_from_dict(alice.preset("2b"))
+    assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.vocab_size, cfg.head_dim) == (26, 2304, 256000, 256)
+    toks = random_tokens(cfg.vocab_size, 300, 62)
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        model = alice.Model.random(cfg, seed=0, dtype=dtype, fast=True)       # the same bfloat16 weights for both paths
+        eng = model.engine(seq_lens=[320], max_seqs=1)
+        s = eng.open(1)
+        got = [eng.step(s, [toks[:292]], "all")] + [eng.step(s, [[t]], "last").clone() for t in toks[292:]]
+        outs[dtype] = torch.cat(got).cpu()
+        del eng, model
+        torch.cuda.empty_cache()
+    f, b = outs["float32"], outs["bfloat16"]
+    assert f.shape == (300, 256000) and 0.5 < float(f.pow(2).mean().sqrt()) < 2.0 and float(f.abs().max()) > 4.0
+    diff = (f - b).abs()
+    assert float(diff.max()) <= 0.06, float(diff.max())
+    assert float(diff.pow(2).mean().sqrt()) < 0.012
+    fa, ba = f.argmax(-1), b.argmax(-1)
+    for p in (fa != ba).nonzero().flatten().tolist():
+        assert float(f[p, fa[p]] - f[p, ba[p]]) < 0.06, p
+    assert int((fa != ba).sum()) <= 3
