@@ -682,6 +682,64 @@ extern "C" int alice_argmax(const float* logits, int* out, float* work_v, int* w
   return 0;
 }
 
+// ---- argmax without a workspace argument
+//
+// The chunk maxima of the two-stage argmax live in a file-scope device array instead of a buffer that the caller
+// allocates.  Every GPU holds its own copy of the array at its own address, which the host learns once per
+// device from hipGetSymbolAddress (in host code the array's name is only a stand-in, not a device address).
+// Nothing in the array has to start at zero: stage one writes every pair that stage two reads.
+static __device__ __align__(256) unsigned char argmax_scratch[ALICE_ARGMAX_STATIC_MAX_PAIRS * 8];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+void* g_argmax_scratch_ptr[MAX_DEVICES] = {};       // per device, set once; a pointer store is atomic on the host
+
+// The address of the current device's copy of the array; nullptr (and the error set) on failure.
+void* argmax_scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    alice_set_error("argmax (static): no current device, or a device number beyond %d", MAX_DEVICES - 1);
+    return nullptr;
+  }
+  void* p = __atomic_load_n(&g_argmax_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p) return p;
+  hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
+  if (e != hipSuccess || !p) {
+    alice_set_error("argmax (static): hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  __atomic_store_n(&g_argmax_scratch_ptr[dev], p, __ATOMIC_RELEASE);   // two threads racing here store the same address
+  return p;
+}
+}  // namespace
+
+extern "C" int alice_argmax_static_init() { return argmax_scratch_of_current_device() ? 0 : 1; }
+
+extern "C" int alice_argmax_static(const float* logits, int* out, int B, int V, hipStream_t stream) {
+  ALICE_CHECK(B >= 0 && V >= 1, "argmax: bad sizes B=%d V=%d", B, V);
+  if (B == 0) return 0;
+  ALICE_CHECK(logits && out, "argmax (static): logits and out must be given");
+  ALICE_CHECK(B <= 65535 * 32, "argmax: too many rows");
+  const int chunks = alice_argmax_chunks(B, V);
+  if (chunks == 1) {
+    argmax_kernel<<<dim3(B, 1), ST, 0, stream>>>(logits, nullptr, out, nullptr, nullptr, V, 1);
+    ALICE_LAUNCH_CHECK();
+    return 0;
+  }
+  ALICE_CHECK((long)B * chunks <= ALICE_ARGMAX_STATIC_MAX_PAIRS,
+              "argmax (static): %d rows in %d chunks need %ld partial results, the static workspace holds %d",
+              B, chunks, (long)B * chunks, ALICE_ARGMAX_STATIC_MAX_PAIRS);
+  void* scratch = argmax_scratch_of_current_device();
+  if (!scratch) return 1;
+  float* work_v = reinterpret_cast<float*>(scratch);
+  int* work_i = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(scratch) + (size_t)ALICE_ARGMAX_STATIC_MAX_PAIRS * 4);
+  argmax_kernel<<<dim3(B, chunks), ST, 0, stream>>>(logits, nullptr, out, work_v, work_i, V, chunks);
+  ALICE_LAUNCH_CHECK();
+  argmax_kernel<<<dim3(B, 1), ST, 0, stream>>>(work_v, work_i, out, nullptr, nullptr, chunks, 1);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
 // Number of 32-bit words of workspace a call needs.
 extern "C" long alice_sample_workspace(int B, int V) {
   int chunks, tiles, per;
