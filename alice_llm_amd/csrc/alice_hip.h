@@ -25,8 +25,6 @@
 #define ALICE_LINEAR_GENERIC 1
 #define ALICE_LINEAR_SKINNY 2
 #define ALICE_LINEAR_MFMA 3
-#define ALICE_LINEAR_TILED256 4   // the tiled kernel with 256 x 256 blocks (MFMA: the 128 x 256 one, or the streaming one)
-#define ALICE_LINEAR_TILED256W8 5 // the same blocks with eight waves (two per SIMD) of 128 x 64 each
 
 #ifdef __cplusplus
 extern "C" {

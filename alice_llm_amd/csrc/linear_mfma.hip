@@ -677,213 +677,6 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
   }
 }
 
-// ---------------------------------------------------------------- tiled, very many tokens: 256 x 256 a block
-// Four waves, two by two: every wave computes 128 tokens x 128 output features as 4 x 4 tiles of the
-// 32x32x16 MFMA (256 accumulator registers per lane), which runs at twice the rate of the 16x16x32 one
-// (measured: 2.1 against 0.8-1.4 PFLOP/s with nothing but MFMAs in the loop).  Both operands go through
-// LDS: a k-tile of the block is 16 token tiles and 16 weight tiles of 1 KB in fragment order, brought by
-// loads that write LDS directly (a lane's 16 bytes land at the tile's base + 16 x lane, which is right for
-// weights, for activations in fragment order and for row-major activations alike), eight tiles per wave.
-// A lane then reads the operand of the wider MFMA from two stacked 16-row tiles: rows lane % 32, inner
-// elements 16 kh + 8 (lane / 32) .. + 7 of k-half kh, i.e. piece (2 kh + lane / 32) * 16 + lane % 16 of tile
-// (lane / 16) % 2.  RING k-tiles are held: while one is multiplied, the fragments of the next are read and
-// the loads of the third after it are issued, and one barrier a k-tile suffices.
-constexpr int RING = 4;
-constexpr int BIG_LDS = RING * 32 * 1024;
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {               // s_waitcnt vmcnt(N), the other counters left alone
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-template <int EPI, typename TO, bool FULL, bool XF, int FI>
-__global__ __launch_bounds__(128 * (8 / FI), 1) void linear_tiled256_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
-                                                                 TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                                 float epi, int gx, int gy, int kt_per_slice, int y_frag,
-                                                                 RopeArgs ra) {
-  extern __shared__ __align__(16) uint32_t ring_raw[];       // [RING][16 token tiles | 2 x 8 weight tiles][64 lanes][16 B]
-  u32x4* ring = reinterpret_cast<u32x4*>(ring_raw);
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int r = lane & 15, g = lane >> 4;
-  const int r32 = lane & 31, h = lane >> 5, upper = (lane >> 4) & 1;
-  constexpr int NW = 2 * (8 / FI), TPW = 32 / NW;            // waves; tiles of a k-tile that a wave brings
-  const int wm = wave & 1, wn = wave >> 1;                   // this wave's half of the tokens, its share of the features
-  const int id = blockIdx.x, xcd = id & 7, local = id >> 3;  // XCD x works through the x-th eighth of the blocks
-  const int per = (gx * gy + 7) >> 3;
-  const int item = xcd * per + local;
-  if (local >= per || item >= gx * gy) return;
-  const int bx = item / gy, by = item % gy;
-  const int m0 = by * 256;
-  // The eight 16-row weight tiles of feature half hf of this block, two stacked per MFMA tile: plainly
-  // consecutive ones, or for GeGLU two of the gate, the same two of the up half, and so on.
-  auto tile_of = [&](int hf, int i) {
-    if (EPI == ALICE_EPI_GEGLU) {
-      const int pair = (bx * 2 + hf) * 4 + 2 * (i >> 2) + (i & 1);
-      return pair >= N / 16 ? NT : (((i >> 1) & 1) ? N / 16 + pair : pair);
-    }
-    return (bx * 2 + hf) * 8 + i;
-  };
-  int tile[2 * FI];                                          // the 16-row weight tiles of this wave's features
-#pragma unroll
-  for (int i = 0; i < 2 * FI; ++i) tile[i] = tile_of((2 * FI * wn + i) >> 3, (2 * FI * wn + i) & 7);
-  // What this wave brings per k-tile: the ring's tiles TPW wave .. + TPW - 1, of which the first 16 are token tiles
-  // and the other 16 the weight tiles of the two feature halves.  One address per tile and lane at k-tile 0; all
-  // loads are unconditional (rows and tiles beyond the matrix are clamped, k-tiles beyond the slice bring the zero
-  // tile or the last k-tile again).
-  const int slot_base = TPW * wave;
-  const bool brings_x = slot_base < 16;
-  const bf16_t* src[TPW];
-#pragma unroll
-  for (int i = 0; i < TPW; ++i) {
-    const int xt = (slot_base + i) & 15, wt = (slot_base + i) & 15;
-    const bf16_t* xs;
-    if constexpr (XF) xs = x + ((size_t)min((m0 >> 4) + xt, (M - 1) >> 4) * KT * 64 + lane) * 8;
-    else xs = x + (size_t)min(m0 + xt * 16 + r, M - 1) * K;
-    const bf16_t* ws = wf + (size_t)min(tile_of(wt >> 3, wt & 7), NT - 1) * KT * 512 + lane * 8;
-    src[i] = brings_x ? xs : ws;
-  }
-  const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
-  const int kt_base = blockIdx.y * kt_per_slice, kt_end = min(KT, kt_base + kt_per_slice);
-  const int T = kt_end - kt_base;
-  y += (size_t)blockIdx.y * M * N;
-  auto bring = [&](int rel) {                                // k-tile kt_base + rel into ring slot rel % RING
-    const int kt = kt_base + rel;
-    const bool kok = kt < kt_end;
-    const int ktc = min(kt, kt_end - 1);
-    size_t off;
-    if (brings_x) off = XF ? (size_t)ktc * 512 : (size_t)min(ktc * 32 + g * 8, K - 8);
-    else off = (size_t)ktc * 512;
-    u32x4* dst = ring + ((size_t)(rel % RING) * 32 + slot_base) * 64;
-#pragma unroll
-    for (int i = 0; i < TPW; ++i) {
-      const bf16_t* p = (brings_x || kok) ? src[i] + off : zero;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
-                                       (__attribute__((address_space(3))) void*)(dst + i * 64), 16, 0, 0);
-    }
-  };
-
-  f32x16 acc[FI][4];                                         // [feature tile of 32][token tile of 32]
-#pragma unroll
-  for (int i = 0; i < FI; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  // Two sets of fragment registers: while the products of k-tile t run on one, the fragments of k-tile t + 1
-  // are read from LDS into the other and the loads of k-tile t + 3 are issued, all between the MFMAs (the
-  // scheduling groups below fix that order; left alone, the compiler puts the reads in front and the wave,
-  // the only one of its SIMD, waits for them).  A k-tile beyond the slice brings zero weights and adds nothing.
-  u32x4 xa[2][4], wa[2][FI], xb[2][4], wb[2][FI];
-  const int piece = h * 16 + r;                              // of k-half 0; k-half 1 is 32 pieces on
-  auto frags = [&](int t, u32x4 (&xf)[2][4], u32x4 (&wk)[2][FI]) {
-    const u32x4* st = ring + (size_t)(t % RING) * 32 * 64;
-#pragma unroll
-    for (int kh = 0; kh < 2; ++kh) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xf[kh][j] = st[(8 * wm + 2 * j + upper) * 64 + kh * 32 + piece];
-#pragma unroll
-      for (int i = 0; i < FI; ++i) wk[kh][i] = st[(16 + 2 * FI * wn + 2 * i + upper) * 64 + kh * 32 + piece];
-    }
-  };
-  auto products = [&](const u32x4 (&xf)[2][4], const u32x4 (&wk)[2][FI]) {
-#pragma unroll
-    for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < FI; ++i) acc[i][j] = mfma32(wk[kh][i], xf[kh][j], acc[i][j]);
-  };
-  auto interleave = [&]() {                                  // 8 FI MFMAs, 8 + 2 FI LDS reads, TPW loads
-#pragma unroll
-    for (int k = 0; k < TPW; ++k) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, FI == 4 ? 1 : 2, 0);
-    }
-  };
-  // A barrier instruction alone: __syncthreads() carries a fence, for which the compiler waits until every
-  // load in flight has written LDS, the ones for the k-tiles ahead included.
-  auto landed = [&]() {
-    wait_vmcnt<(RING - 2) * TPW>();                            // all but the newest RING - 2 k-tiles asked for: this wave's part is there
-    asm volatile("s_barrier" ::: "memory");                  // everyone's is, and everyone is done with the k-tile before
-  };
-  // During the products of k-tile t (fragments in registers) the ring holds k-tile t + 1, which is being read,
-  // and the RING - 1 after it, which are on their way: k-tile t + RING goes where k-tile t was.
-#pragma unroll
-  for (int s = 0; s < RING; ++s) bring(s);
-  wait_vmcnt<(RING - 1) * TPW>();
-  asm volatile("s_barrier" ::: "memory");
-  frags(0, xa, wa);
-  for (int t = 0; t < T; t += 2) {
-    landed();                                                // k-tile t + 1
-    bring(t + RING);
-    frags(t + 1, xb, wb);
-    products(xa, wa);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    landed();                                                // k-tile t + 2
-    bring(t + 1 + RING);
-    frags(t + 2, xa, wa);
-    products(xb, wb);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  wait_vmcnt<0>();                                           // the loads past the end still write LDS
-
-  // Lane l of an accumulator holds, for token 32 j + l % 32, features 8 q + 4 (l / 32) + e (q, e < 4) of the
-  // 32 of MFMA tile i: four consecutive ones per q, in 16-row tile 2 i + q / 2 of the wave's eight.
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int m = m0 + (8 * wm) * 16 + 32 * j + r32;
-    if (m >= M) continue;
-    const size_t row_off = (size_t)m * N;
-    if constexpr (EPI == ALICE_EPI_ROPE) {
-      const RopeToken tk = rope_token(ra, m);
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t16 = tile[2 * i + (q >> 1)];
-          if (t16 >= NT) continue;
-          const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          rope_store4(ra, m, tk, t16 * 16 + 8 * (q & 1) + 4 * h, v);
-        }
-    } else if constexpr (EPI == ALICE_EPI_GEGLU) {
-#pragma unroll
-      for (int p = 0; p < FI / 2; ++p)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t16 = tile[4 * p + (q >> 1)];            // the gate's tile; the up half's has the same place in N
-          if (t16 >= NT) continue;
-          f32x4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][4 * q + e], FULL) * acc[2 * p + 1][j][4 * q + e];
-          store4_any(y, y_frag, m, row_off, t16 * 16 + 8 * (q & 1) + 4 * h, N, o);
-        }
-    } else {
-#pragma unroll
-      for (int i = 0; i < FI; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t16 = tile[2 * i + (q >> 1)];
-          if (t16 >= NT) continue;
-          f32x4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][4 * q + e], epi);
-          store4_any(y, y_frag, m, row_off, t16 * 16 + 8 * (q & 1) + 4 * h, N, o);
-        }
-    }
-  }
-}
-
 // ---------------------------------------------------------------- layout conversion
 __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N, int K, int KT, size_t total) {
   const size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x;     // index in dst, in elements
@@ -913,9 +706,20 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
   // k-tiles per wave, and whether windows of five waste fewer slots than windows of four (see the kernel)
   const int nw = eight ? 8 : 4, J = ceil_div(min(per, KT), nw);
   const bool five = RT * MT <= 2 && x_frag && (ceil_div(J, 5) * 5 - J) < (ceil_div(J, 4) * 4 - J);
+  // The reduction's LDS passes 64 KB with six row tiles and four token tiles: the kernel is told once.
 #define SKINNY(NWV, THREADS, XFV, STREAMV, WINV)                                                                             \
-  linear_skinny_kernel<RT, MT, NWV, EPI, TO, false, XFV, STREAMV, WINV><<<grid, THREADS, lds, s>>>(                           \
-      (const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra)
+  do {                                                                                                                         \
+    auto kern = linear_skinny_kernel<RT, MT, NWV, EPI, TO, false, XFV, STREAMV, WINV>;                                        \
+    if (lds > 48 * 1024) {                                                                                                     \
+      static bool told = false;                                                                                                \
+      if (!told) {                                                                                                             \
+        ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, \
+                    "linear: the device does not give a block %d bytes of LDS", (int)lds);                                     \
+        told = true;                                                                                                           \
+      }                                                                                                                        \
+    }                                                                                                                          \
+    kern<<<grid, THREADS, lds, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, per, epi, y_frag, ra);       \
+  } while (0)
 #define BY_INPUT(NWV, THREADS)                                                        \
   do {                                                                                \
     if constexpr (RT * MT <= 2) {                                                     \
@@ -942,13 +746,39 @@ int launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, in
 // Row tiles per block: few keep the chip full on narrow matrices, more amortise the activation reads
 // on wide ones.  (GeGLU needs an even number: gate and up tiles come in pairs.)  Measured on the 2B
 // shapes with the activations in fragment order.
-int skinny_row_tiles(int M, int N, int epi, int split, int K) {
+int skinny_row_tiles_base(int M, int N, int epi, int split, int K) {
   const int tiles = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   if (tiles >= 4096) return 4;
   if (epi == ALICE_EPI_GEGLU) return 2;
   // Many tokens and slices of the inner dimension: more rows per block per read of the activations.
   if (M > 32 && split > 1 && tiles >= 64) return K >= 8192 ? 4 : 2;
   return tiles >= 1024 ? 2 : 1;
+}
+
+// What a choice of row tiles and slices costs, in units of one k-tile of one row tile read by a CU: the busiest of
+// the 256 CUs runs ceil(blocks / 256) blocks one after the other (or side by side, sharing what it can load), each
+// reading rt weight tiles and the token tiles' activations (which come from the L2: half the price) per k-tile,
+// and every slice adds a partial result and shortens each wave's run.  Fitted to the 2B, 9B and 27B matrices at 1
+// to 64 tokens: gate/up of the 2B shape at 64 tokens takes 27.5, 30.5 and 22.9 us with 2, 4 and 6 row tiles (576,
+// 288 and 192 blocks: 3, 2 and 1 per CU), the 9B shape 57.5, 49.6 and 58.7 us, the 27B shape 168, 148 and 132 us.
+float skinny_cost(int M, int N, int K, int epi, int rt, int split) {
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4), KT = (K + 31) / 32;
+  const int groups = epi == ALICE_EPI_GEGLU ? ceil_div(N / 16, rt / 2) : ceil_div(ceil_div(N, 16), rt);
+  return (float)ceil_div((long)groups * split, 256) * ceil_div(KT, split) * (rt + 0.5f * mt) + 20.f * split;
+}
+
+// Six row tiles a block where the cost above says so: gate/up by the cost alone, the other products only where
+// six beat the rule above by 7 % (that rule is measured, the cost is a model).
+int skinny_row_tiles(int M, int N, int epi, int split, int K) {
+  const int base = skinny_row_tiles_base(M, N, epi, split, K);
+  if (epi == ALICE_EPI_GEGLU) {
+    int best = 2;
+    for (int rt = 4; rt <= 6; rt += 2)
+      if (skinny_cost(M, N, K, epi, rt, 1) < skinny_cost(M, N, K, epi, best, 1)) best = rt;
+    return best;
+  }
+  if (epi != ALICE_EPI_NONE) return base;
+  return skinny_cost(M, N, K, epi, 6, split) < 0.93f * skinny_cost(M, N, K, epi, base, split) ? 6 : base;
 }
 
 template <int EPI, typename TO>
@@ -958,6 +788,7 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
 #define GO(RT, MT) return launch_skinny<RT, MT, EPI, TO>(x, w, y, M, N, K, split, epi, x_frag, y_frag, s)
 #define BY_RT(MT)                                                   \
   do {                                                              \
+    if constexpr (EPI != ALICE_EPI_SOFTCAP) { if (rt == 6) GO(6, MT); } \
     if (rt == 4) GO(4, MT);                                         \
     if (rt == 2) GO(2, MT);                                         \
     if constexpr (EPI != ALICE_EPI_GEGLU) GO(1, MT);                \
@@ -970,41 +801,11 @@ int skinny_by_shape(const void* x, const void* w, void* y, int M, int N, int K, 
   return 1;
 }
 
-// Whether the 256 x 256 blocks are worth it.  Not yet: with one wave per SIMD the waits for LDS and for the
-// barrier are not hidden, and the kernel runs at 0.8 of the speed of the 128 x 256 one; it is reached by its
-// variant only.
-inline bool big_tiles_pay(int, int, int) { return false; }
-
 template <int EPI, typename TO>
 int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
-                 hipStream_t s, const RopeArgs& ra = RopeArgs{}, int big = 0) {
+                 hipStream_t s, const RopeArgs& ra = RopeArgs{}) {
   const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
   const int per = ceil_div(KT, split);
-  {
-    // big: 1 forces the 256 x 256 blocks with four waves, 2 with eight, -1 forbids them
-    const int gx256 = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 8) : ceil_div(NT, 16);
-    if (big > 0 || (big == 0 && big_tiles_pay(M, gx256, split))) {
-      const int gy256 = ceil_div(M, 256);
-      dim3 grid(8 * ceil_div(gx256 * gy256, 8), split);
-      auto go = [&](auto kern, int threads, bool& prepared) {
-        if (!prepared) {
-          if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BIG_LDS) != hipSuccess) return false;
-          prepared = true;
-        }
-        kern<<<grid, threads, BIG_LDS, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx256, gy256, per, y_frag, ra);
-        return true;
-      };
-      static bool prepared[4] = {false, false, false, false};
-      bool ok;
-      if (big == 2) ok = x_frag ? go(linear_tiled256_kernel<EPI, TO, false, true, 2>, 512, prepared[3])
-                                : go(linear_tiled256_kernel<EPI, TO, false, false, 2>, 512, prepared[2]);
-      else ok = x_frag ? go(linear_tiled256_kernel<EPI, TO, false, true, 4>, 256, prepared[1])
-                       : go(linear_tiled256_kernel<EPI, TO, false, false, 4>, 256, prepared[0]);
-      ALICE_CHECK(ok, "linear: the device does not give a block %d bytes of LDS", BIG_LDS);
-      ALICE_LAUNCH_CHECK();
-      return 0;
-    }
-  }
   const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
   int gy = ceil_div(M, 16 * WM);
   // 128 tokens a block, or 64 when that leaves most of the chip without a block (measured at N = 2304 and 4096:
@@ -1042,6 +843,23 @@ extern "C" int alice_to_frag16(const void* src, void* dst, int N, int K, hipStre
   return 0;
 }
 
+// The number of slices once six row tiles a block are a choice: half or twice the measured rule's number where the
+// cost (with the row tiles that skinny_row_tiles would then pick) is 7 % lower.
+static int skinny_split_with_six(int M, int N, int K, int split0) {
+  const int KT = (K + 31) / 32;
+  auto cost_at = [&](int sp) {
+    return skinny_cost(M, N, K, ALICE_EPI_NONE, skinny_row_tiles(M, N, ALICE_EPI_NONE, sp, K), sp);
+  };
+  int best = split0;
+  float best_cost = cost_at(split0) * 0.93f;
+  for (int sp : {split0 / 2, split0 * 2}) {
+    if (sp < 1 || sp > 16 || sp == split0 || (sp > 1 && KT / sp < 16)) continue;
+    const float c = cost_at(sp);
+    if (c < best_cost) { best_cost = c; best = sp; }
+  }
+  return best;
+}
+
 int alice_linear_split_hint_frag(int M, int N, int K) {
   if (M > 64) {
     // Tiled kernel: 128 tokens x 256 features a block, two blocks a CU.  Narrow outputs leave most of the
@@ -1062,12 +880,12 @@ int alice_linear_split_hint_frag(int M, int N, int K) {
     return best;
   }
   const int KT = (K + 31) / 32;
-  if (M > 32) return KT >= 128 ? 4 : (KT >= 32 ? 2 : 1);
-  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles(M, N, ALICE_EPI_NONE, 1, K));
+  if (M > 32) return skinny_split_with_six(M, N, K, KT >= 128 ? 4 : (KT >= 32 ? 2 : 1));
+  const int groups = ceil_div(ceil_div(N, 16), skinny_row_tiles_base(M, N, ALICE_EPI_NONE, 1, K));
   int split = 1;
   // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
   while (groups * split < 1024 && KT / (split * 2) >= 16 && split < 16) split *= 2;
-  return split;
+  return skinny_split_with_six(M, N, K, split);
 }
 
 int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_dtype, int M, int N, int K,
@@ -1107,8 +925,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
     }                                                                                              \
   } while (0)
   if (skinny) BY_EPI(skinny_by_shape, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream);
-  const int big = variant == ALICE_LINEAR_TILED256 ? 1 : variant == ALICE_LINEAR_TILED256W8 ? 2 : (variant == ALICE_LINEAR_MFMA ? -1 : 0);
-  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream, RopeArgs{}, big);
+  BY_EPI(launch_tiled, x, w, y, M, N, K, split_k, epi_param, x_frag, y_frag, stream, RopeArgs{});
 #undef BY_EPI
 }
 

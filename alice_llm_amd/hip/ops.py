@@ -17,7 +17,7 @@ from ..csrc import build as _build
 
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
-LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED256, LINEAR_TILED256W8 = 0, 1, 2, 3, 4, 5
+LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA = 0, 1, 2, 3
 ABI_VERSION = 4
 
 _lib = None

@@ -443,49 +443,25 @@ def test_linear_mfma(M, N, K, ydt):
             close(yp.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 32), (300, 1000, 416), (1000, 80, 2048), (513, 528, 72), (70, 304, 160)])
-@pytest.mark.parametrize("waves", [4, 8])
-def test_linear_mfma_blocks_of_256(M, N, K, waves):
-    """The kernel with 256 x 256 blocks (four waves of 128 x 128, or eight of 128 x 64), forced, against the plain product (its MFMA adds 16 inner elements at a
-    time, the other kernels' 32: the same sums in another order)."""
-    big = ops.LINEAR_TILED256 if waves == 4 else ops.LINEAR_TILED256W8
-    x, w = rnd(M, K, seed=70, dtype=torch.bfloat16), rnd(N, K, seed=71, scale=0.1, dtype=torch.bfloat16)
-    wf = ops.to_frag16(w)
-    ref = x.double() @ w.double().T
-    for ydt, atol, rtol in ((torch.float32, 2e-4, 1e-5), (torch.bfloat16, 1e-2, 2 ** -8)):
-        y, y0 = (torch.full((M, N), float("nan"), dtype=ydt, device=DEV) for _ in range(2))
-        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=big, full_precision=False)
-        ops.linear(x, wf, y0, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_MFMA, full_precision=False)
-        close(y, ref, atol * math.sqrt(K / 64), rtol)
-        close(y0, ref, atol * math.sqrt(K / 64), rtol)
-    y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
-    ops.linear(x, wf, y2, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_SOFTCAP, epi_param=3.0,
-               variant=big, full_precision=False)
-    close(y2, 3.0 * torch.tanh(ref / 3.0), 1e-3)
-    for split in (2, 3):
-        if K // 32 >= split:
-            yp = torch.full((split, M, N), float("nan"), dtype=torch.float32, device=DEV)
-            ops.linear(x, wf, yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=big,
-                       full_precision=False)
-            close(yp.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
-    if K % 32 == 0:
-        yf = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.linear(acts_to_fragments(x), wf, yf, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=big,
-                   full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16)
-        assert torch.equal(yf, y)                          # the same bits from rows and from fragments
-    if N % 32 == 0:
-        flat = torch.full(((-(-M // 16) * 16) * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.linear(x, wf, flat, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=big, full_precision=False,
-                   rows=M, y_layout=ops.LAYOUT_FRAG16)
-        assert torch.equal(acts_from_fragments(flat, M, N), y.cpu())
-    if N % 16 == 0:
-        w2 = rnd(2 * N, K, seed=72, scale=0.3, dtype=torch.bfloat16)
-        wf2 = ops.to_frag16(w2)
-        gate, up = x.double() @ w2.double()[:N].T, x.double() @ w2.double()[N:].T
-        yg = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.linear(x, wf2, yg, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, variant=big,
-                   full_precision=False)
-        close(yg, F.gelu(gate, approximate="tanh") * up, 2e-2, 2 ** -7)
+@pytest.mark.parametrize("M", [3, 20, 40, 64])
+def test_linear_streaming_with_six_row_tiles(M):
+    """Shapes for which the streaming kernel takes six row tiles a block (the cost rule of the launcher picks them
+    where three blocks' worth of tiles would otherwise wait for one another), with tile counts that six does not
+    divide: gate/up of 577 pairs, and a product of 145 row tiles in slices of the inner dimension."""
+    K = 512
+    x = rnd(M, K, seed=80, dtype=torch.bfloat16)
+    w2 = rnd(2 * 9232, K, seed=81, scale=0.3, dtype=torch.bfloat16)
+    gate, up = x.double() @ w2.double()[:9232].T, x.double() @ w2.double()[9232:].T
+    yg = torch.full((M, 9232), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, ops.to_frag16(w2), yg, n_out=9232, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU, full_precision=False)
+    close(yg, F.gelu(gate, approximate="tanh") * up, 2e-2, 2 ** -7)
+    N, K = 2320, 9216
+    x, w = rnd(M, K, seed=82, dtype=torch.bfloat16), rnd(N, K, seed=83, scale=0.1, dtype=torch.bfloat16)
+    split = ops.linear_split_hint(M, N, K, ops.LAYOUT_FRAG16)
+    assert split > 1
+    yp = torch.full((split, M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.linear(x, ops.to_frag16(w), yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False)
+    close(yp.sum(0), x.double() @ w.double().T, 2e-4 * math.sqrt(K / 64), 1e-5)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 48, 96), (200, 304, 96), (129, 2048, 64)])
