@@ -38,6 +38,9 @@ class Gemma2Config:
     eos_token_id: Tuple[int, ...] = (1,)
     bos_token_id: Optional[int] = 2
     torch_dtype: str = "bfloat16"
+    # Which layers slide, when config.json says so layer by layer ("sliding_attention" / "full_attention");
+    # absent: even layers slide and odd layers see everything, the rule the reference has in code (llama3.rs:4634-4641).
+    layer_types: Optional[Tuple[str, ...]] = None
 
     architecture = "Gemma2ForCausalLM"
     model_type = "gemma2"
@@ -68,6 +71,11 @@ class Gemma2Config:
             eos = ()
         else:
             raise ConfigError(f"config.json: key 'eos_token_id' must be an integer or a list of integers, found {eos!r}")
+        kinds = d.get("layer_types")
+        if kinds is not None:
+            if not isinstance(kinds, (list, tuple)) or not all(isinstance(k, str) for k in kinds):
+                raise ConfigError(f"config.json: key 'layer_types' must be a list of strings, found {kinds!r}")
+            kinds = tuple(kinds)
         cfg = cls(
             vocab_size=V, hidden_size=H, num_hidden_layers=L, num_attention_heads=nH,
             num_key_value_heads=nKV, head_dim=hd, intermediate_size=I,
@@ -83,7 +91,8 @@ class Gemma2Config:
             tie_word_embeddings=read_key(d, "tie_word_embeddings", bool, True),
             eos_token_id=eos,
             bos_token_id=read_key(d, "bos_token_id", int, 2, allow_none=True),
-            torch_dtype=read_key(d, "torch_dtype", str, "bfloat16"),
+            torch_dtype=read_key(d, "torch_dtype", str, read_key(d, "dtype", str, "bfloat16")),
+            layer_types=kinds,
         )
         cfg.validate()
         return cfg
@@ -106,6 +115,11 @@ class Gemma2Config:
         require(self.query_pre_attn_scalar > 0, "query_pre_attn_scalar must be positive")
         require(self.hidden_activation == "gelu_pytorch_tanh",
                 f"hidden_activation must be 'gelu_pytorch_tanh' for Gemma 2, found '{self.hidden_activation}'")
+        if self.layer_types is not None:
+            require(len(self.layer_types) == self.num_hidden_layers,
+                    f"layer_types names {len(self.layer_types)} layers, num_hidden_layers is {self.num_hidden_layers}")
+            bad = sorted(set(self.layer_types) - {"sliding_attention", "full_attention"})
+            require(not bad, f"layer_types holds {bad}: only 'sliding_attention' and 'full_attention' have a kernel")
         require(self.torch_dtype in ("bfloat16", "float32"),
                 f"torch_dtype must be 'bfloat16' or 'float32', found '{self.torch_dtype}'")
 
@@ -114,6 +128,10 @@ class Gemma2Config:
         d["architectures"] = [self.architecture]
         d["model_type"] = self.model_type
         d["eos_token_id"] = list(self.eos_token_id) if len(self.eos_token_id) != 1 else self.eos_token_id[0]
+        if self.layer_types is None:
+            del d["layer_types"]
+        else:
+            d["layer_types"] = list(self.layer_types)
         return d
 
     # ------------------------------------------------------------------ derived
@@ -126,7 +144,9 @@ class Gemma2Config:
         return self.num_key_value_heads * self.head_dim
 
     def layer_window(self, i: int) -> Optional[int]:
-        """Even layers slide, odd layers are global (llama3.rs:4636-4641)."""
+        """Even layers slide, odd layers are global (llama3.rs:4636-4641), unless layer_types says otherwise."""
+        if self.layer_types is not None:
+            return self.sliding_window if self.layer_types[i] == "sliding_attention" else None
         return self.sliding_window if i % 2 == 0 else None
 
     # ------------------------------------------------------------------ the plan

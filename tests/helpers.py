@@ -27,7 +27,12 @@ TINY_C = dict(_COMMON, num_hidden_layers=4, hidden_size=160, num_attention_heads
               head_dim=64, intermediate_size=416, vocab_size=1000, rope_theta=20000.0, sliding_window=80,
               query_pre_attn_scalar=48, attn_logit_softcapping=12.0, final_logit_softcapping=9.0,
               rms_norm_eps=2e-6, max_position_embeddings=1024)
-TINY = {"tiny-a": (TINY_A, 0), "tiny-b": (TINY_B, 1), "tiny-c": (TINY_C, 2)}
+# The options that the published Gemma 2 configurations leave at their defaults, all turned the other way: a head with
+# a matrix of its own, no caps, and the layers' kinds listed in config.json (global first, then two sliding layers).
+TINY_D = dict(TINY_B, tie_word_embeddings=False, attn_logit_softcapping=None, final_logit_softcapping=None,
+              layer_types=["full_attention", "sliding_attention", "sliding_attention"], sliding_window=5, hidden_size=80,
+              num_attention_heads=4, num_key_value_heads=4, head_dim=32, query_pre_attn_scalar=32, vocab_size=130)
+TINY = {"tiny-a": (TINY_A, 0), "tiny-b": (TINY_B, 1), "tiny-c": (TINY_C, 2), "tiny-d": (TINY_D, 3)}
 
 _FOLDERS = {}
 _TMP = None

@@ -148,6 +148,7 @@ class PlainGemma2:
         self.cap_a = c.get("attn_logit_softcapping", 50.0)
         self.cap_f = c.get("final_logit_softcapping", 30.0)
         self.scale = float(c.get("query_pre_attn_scalar", self.d)) ** -0.5
+        self.layer_types = c.get("layer_types")
         self.t = {k: v.to(dtype) for k, v in tensors.items()}
 
     @classmethod
@@ -162,7 +163,10 @@ class PlainGemma2:
         return cls(config, tensors, dtype, dense)
 
     def layer_window(self, i: int):
-        """Even layers slide, odd layers see everything.  llama3.rs:4634-4641."""
+        """Even layers slide, odd layers see everything (llama3.rs:4634-4641); a config.json that lists
+        layer_types layer by layer overrides the rule."""
+        if self.layer_types is not None:
+            return self.window if self.layer_types[i] == "sliding_attention" else None
         return self.window if i % 2 == 0 else None
 
     def embed(self, tokens):

@@ -46,6 +46,7 @@ def test_config_defaults_and_nulls():
     ({"final_logit_softcapping": -1.0}, "final_logit_softcapping"), ({"hidden_activation": "silu"}, "gelu_pytorch_tanh"),
     ({"architectures": ["LlamaForCausalLM"]}, "registered"), ({"num_hidden_layers": True}, "integer"),
     # keys that would change the arithmetic and that nothing implements are refused, not dropped
+    ({"layer_types": ["sliding_attention"]}, "layer_types names 1"), ({"layer_types": ["full_attention", "chunked"]}, "chunked"),
     ({"attention_bias": True}, "attention_bias"), ({"rope_scaling": {"type": "linear", "factor": 2.0}}, "rope_scaling"),
 ])
 def test_config_errors_name_the_key(change, word):
@@ -57,6 +58,12 @@ def test_config_errors_name_the_key(change, word):
             d[k] = v
     with pytest.raises(ConfigError, match=word):
         alice.config_from_dict(d)
+
+
+def test_layer_kinds_from_config_when_it_lists_them():
+    c = alice.config_from_dict(dict(TINY_B, layer_types=["full_attention", "sliding_attention", "sliding_attention"], dtype="float32"))
+    assert [l.mixer.args["window"] for l in c.plan().layers] == [None, 6, 6] and c.torch_dtype == "float32"
+    assert alice.config_from_dict(c.to_dict()) == c and "layer_types" not in alice.config_from_dict(dict(TINY_B)).to_dict()
 
 
 def test_registry(tmp_path):

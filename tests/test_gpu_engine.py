@@ -8,7 +8,7 @@ from helpers import TINY, TOL, max_err, model_folder, plain_model, random_tokens
 
 pytestmark = pytest.mark.gpu
 
-CASES = [(n, d) for n in ("tiny-a", "tiny-b", "tiny-c") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("tiny-a", "tiny-b", "tiny-c", "tiny-d") for d in ("float32", "bfloat16")]
 _MODELS = {}
 
 

@@ -102,3 +102,24 @@ def test_replay_without_wanted_logits_writes_nothing(tmp_path):
     plain = plain_model(folder)
     got = torch.from_numpy(np.fromfile(out / "1.f32", dtype="<f4").copy())
     assert (got.double() - plain.forward([1, 2, 3, 4])[-1]).abs().max() < TOL["float32"]
+
+
+def test_replay_bad_input_ends_with_one_line(tmp_path):
+    folder = model_folder("tiny-a", "bfloat16")
+    run = lambda text, model=folder: subprocess.run(
+        [os.path.join(ROOT, "bin", "trace_run"), "--model", model, "--dtype", "float32", "--out", str(tmp_path / "o"),
+         "--max-tokens", "64"], input=text, capture_output=True, text=True, timeout=300)
+    ok = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [1, 2], "want": [1]}], "end": []})
+    cases = [("{not json\n", "input line 1"),
+             (ok + "\n" + json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [999], "want": [0]}], "end": []}) + "\n", "step 1.*vocabulary"),
+             (ok + "\n" + json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [3], "want": [4]}], "end": []}) + "\n", "step 1.*want"),
+             (ok + "\n" + json.dumps({"step": 1, "entries": [{"id": "a", "want": [0]}], "end": []}) + "\n", "step 1.*tokens"),
+             (json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [1] * 70, "want": []}], "end": []}) + "\n", "step 0.*full")]
+    import re
+    for text, pattern in cases:
+        proc = run(text)
+        lines = [l for l in proc.stderr.splitlines() if l.startswith("trace_run:")]
+        assert proc.returncode == 1 and len(lines) == 1 and re.search(pattern, lines[0]), (pattern, proc.stderr[-500:])
+        assert "Traceback" not in proc.stderr
+    proc = run(ok + "\n", model=str(tmp_path / "nowhere"))
+    assert proc.returncode == 1 and "cannot load" in proc.stderr and "Traceback" not in proc.stderr
