@@ -25,6 +25,8 @@
 #define ALICE_LINEAR_GENERIC 1
 #define ALICE_LINEAR_SKINNY 2
 #define ALICE_LINEAR_MFMA 3
+#define ALICE_LINEAR_TILED_W16 4   // the tiled kernel with a wave tile of 16 output features (activations in fragment order)
+#define ALICE_LINEAR_TILED_W32 5   // the same with 32
 
 #ifdef __cplusplus
 extern "C" {

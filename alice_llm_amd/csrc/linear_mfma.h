@@ -199,10 +199,17 @@ int alice_mfma_stream(const void* x, const void* w, void* y, int y_dtype, int M,
                       int split, int x_frag, int y_frag, hipStream_t s);
 // The same with the rotation and the cache write as its epilogue.
 int alice_mfma_stream_rope(const void* x, const void* w, int M, int N, int K, int x_frag, hipStream_t s, const RopeArgs& ra);
-// The tiled kernel (many tokens), and with the rotation epilogue.
+// The tiled kernel (many tokens), and with the rotation epilogue.  force_wn 1 or 2: the wave tile of 16 or 32
+// features whatever the cost rule says (0: the rule's choice).
 int alice_mfma_tiled(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K, int epi, float epi_param,
-                     int split, int x_frag, int y_frag, hipStream_t s);
+                     int split, int x_frag, int y_frag, int force_wn, hipStream_t s);
 int alice_mfma_tiled_rope(const void* x, const void* w, int M, int N, int K, int x_frag, hipStream_t s, const RopeArgs& ra);
+// The tiled kernel's tile: a wave's 16 wn output features x 16 tm tokens, kc k-tiles a stage, slices of the inner
+// dimension.  split 0: the rule chooses the slices too (float32 sums without epilogue only), else they are given.
+struct TiledPlan { int wn, tm, kc, split; };
+TiledPlan alice_mfma_tiled_plan(int M, int N, int K, int epi, int y_dtype, int split, int x_frag);
+int alice_mfma_tiled_narrow(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K, int epi, float epi_param,
+                            const TiledPlan& p, int y_frag, hipStream_t s, const RopeArgs& ra);
 // The streaming kernel's choice of row tiles a block and what the launcher's cost rule says of a choice.
 int alice_mfma_stream_row_tiles(int M, int N, int epi, int split, int K);
 int alice_mfma_stream_row_tiles_base(int M, int N, int epi, int split, int K);

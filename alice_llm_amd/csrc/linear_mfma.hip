@@ -58,24 +58,8 @@ static int skinny_split_with_six(int M, int N, int K, int split0) {
 }
 
 int alice_linear_split_hint_frag(int M, int N, int K) {
-  if (M > 64) {
-    // Tiled kernel: 128 tokens x 256 features a block, two blocks a CU.  Narrow outputs leave most of the
-    // chip idle; slices of the inner dimension fill it.  Cost of s slices, relative to one block a CU
-    // running the whole inner dimension: the busiest CU runs n = ceil(blocks s / 256) blocks of 1/s the
-    // length, two at a time at 1.7 times the time of one; every extra slice writes and reads another
-    // [M, N] float32 partial result (both constants fitted to measurements at N = 2304, K = 2048 and 9216).
-    const int blocks = ceil_div(N, 256) * ceil_div(M, 128), KT = (K + 31) / 32;
-    if (blocks >= 384) return 1;
-    int best = 1;
-    float best_cost = 1e30f;
-    for (int s = 1; s <= 6; ++s) {
-      if (s > 1 && KT / s < 16) break;
-      const int n = ceil_div(blocks * s, 256);
-      const float cost = (1.7f * (n / 2) + (n % 2)) / s + 3.6f * blocks / K * (s - 1);
-      if (cost < best_cost * 0.97f) { best_cost = cost; best = s; }
-    }
-    return best;
-  }
+  // more than 64 tokens: the tiled kernel's own rule (activations in fragment order, as prompts bring them)
+  if (M > 64) return alice_mfma_tiled_plan(M, N, K, ALICE_EPI_NONE, DT_F32, 0, 1).split;
   const int KT = (K + 31) / 32;
   if (M > 32) return skinny_split_with_six(M, N, K, KT >= 128 ? 4 : (KT >= 32 ? 2 : 1));
   const int groups = ceil_div(ceil_div(N, 16), alice_mfma_stream_row_tiles_base(M, N, ALICE_EPI_NONE, 1, K));
@@ -110,7 +94,8 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
               "linear: output in fragment order needs bfloat16, N %% 32 == 0, no softcap and no partial sums");
   const int x_frag = x_layout == ALICE_LAYOUT_FRAG16, y_frag = y_layout == ALICE_LAYOUT_FRAG16;
   if (skinny) return alice_mfma_stream(x, w, y, y_dtype, M, N, K, epi, epi_param, split_k, x_frag, y_frag, stream);
-  return alice_mfma_tiled(x, w, y, y_dtype, M, N, K, epi, epi_param, split_k, x_frag, y_frag, stream);
+  const int force_wn = variant == ALICE_LINEAR_TILED_W16 ? 1 : variant == ALICE_LINEAR_TILED_W32 ? 2 : 0;
+  return alice_mfma_tiled(x, w, y, y_dtype, M, N, K, epi, epi_param, split_k, x_frag, y_frag, force_wn, stream);
 }
 
 extern "C" int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, int K, void* q_out, void* k_pool,

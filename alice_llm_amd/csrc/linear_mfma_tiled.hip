@@ -1,351 +1,110 @@
-// The tiled matrix product for many tokens (prompts) on the matrix cores; the layouts and the operand roles are
-// described in linear_mfma.h.  y[r] = sum_c W[r,c] x[c] (gguf.rs:4063-4074) with the GeGLU (llama3.rs:14519-14534),
-// softcap (llama3.rs:14606-14611) and rotation (llama3.rs:5367-5378) epilogues.
-#include "linear_mfma.h"
+// The tiled matrix product for many tokens: the choice of its tile (wave tile width, tokens a block, k-tiles a stage,
+// slices of the inner dimension) and the launches with the widest wave tile; the kernel is in linear_mfma_tiled.h, the
+// launches with narrower tiles in linear_mfma_tiled_narrow.hip.
+#include "linear_mfma_tiled.h"
 
 namespace {
 
-constexpr int WM = 8, WN = 4;   // a wave's tile: 8 x 4 MFMA tiles = 128 tokens x 64 output features
+// Slices of the inner dimension for the widest tile: 128 tokens x 256 features a block, two blocks a CU.  Narrow
+// outputs leave most of the chip idle; slices fill it.  Cost of s slices, relative to one block a CU running the
+// whole inner dimension: the busiest CU runs n = ceil(blocks s / 256) blocks of 1/s the length, two at a time at
+// 1.7 times the time of one; every extra slice writes and reads another [M, N] float32 partial result (both
+// constants fitted to measurements at N = 2304, K = 2048 and 9216).
+int tiled_split_wide(int M, int N, int K) {
+  const int blocks = ceil_div(N, 256) * ceil_div(M, 128), KT = (K + 31) / 32;
+  if (blocks >= 384) return 1;
+  int best = 1;
+  float best_cost = 1e30f;
+  for (int s = 1; s <= 6; ++s) {
+    if (s > 1 && KT / s < 16) break;
+    const int n = ceil_div(blocks * s, 256);
+    const float cost = (1.7f * (n / 2) + (n % 2)) / s + 3.6f * blocks / K * (s - 1);
+    if (cost < best_cost * 0.97f) { best_cost = cost; best = s; }
+  }
+  return best;
+}
 
-// ---------------------------------------------------------------- tiled, many tokens
-// Block: 4 waves side by side along N; every wave computes 128 (or 64) tokens x 64 output features
-// (8 x 4 MFMA tiles, 128 accumulator registers per lane) and streams its own weight tiles straight
-// from memory.  The block's tokens x 64 inner elements of activations are staged once in LDS (in
-// fragment order, so LDS reads and writes are linear) and read by all four waves.  Two stages are kept: while one is used for the
-// MFMAs the next one's global loads are in flight, and one barrier per stage suffices.  The grid is
-// one-dimensional and mapped so that the blocks that share weight tiles run on the same XCD (blocks
-// are dealt to the eight XCDs round robin by their linear index).
-constexpr int KC = 2;      // k-tiles per stage
-
-// XF: the activations come in fragment order (a compile-time choice: as a run-time one it cost the
-// row-major path a third of its speed).
-template <int EPI, typename TO, bool FULL, int TM, bool XF>
-__global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wf,
-                                                               TO* __restrict__ y, int M, int N, int K, int KT, int NT,
-                                                               float epi, int gx, int gy, int kt_per_slice, int y_frag,
-                                                               RopeArgs ra) {
-  constexpr int XJ = TM / 4;                               // token tiles each wave stages
-  // The rotation epilogue stages 64 tokens x 256 features in the same memory afterwards (ROPE_PITCH elements a token).
-  constexpr int XS_WORDS = 2 * KC * TM * 64 * 4;
-  constexpr int LDS_WORDS = (EPI == ALICE_EPI_ROPE && XS_WORDS < 64 * ROPE_PITCH / 2) ? 64 * ROPE_PITCH / 2 : XS_WORDS;
-  __shared__ __align__(16) uint32_t xs_raw[LDS_WORDS];
-  u32x4* xs = reinterpret_cast<u32x4*>(xs_raw);            // [2][KC][TM][64]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  // Blocks go to the XCDs round robin by index; XCD x works through the x-th eighth of the tiles in
-  // column-major order, so that tiles with the same weight columns meet in one L2.
-  const int id = blockIdx.x, xcd = id & 7, local = id >> 3;
-  const int per = (gx * gy + 7) >> 3;
-  const int item = xcd * per + local;
-  if (local >= per || item >= gx * gy) return;
-  const int bx = item / gy, by = item % gy;
-  const int m0 = by * (16 * TM);
-  int tile[WN];
-#pragma unroll
-  for (int i = 0; i < WN; ++i) {
-    if (EPI == ALICE_EPI_GEGLU) {
-      const int pair = (bx * 4 + wave) * (WN / 2) + (i >> 1);
-      tile[i] = (i & 1) ? N / 16 + pair : pair;
-      if (pair >= N / 16) tile[i] = NT;
-    } else {
-      tile[i] = (bx * 4 + wave) * WN + i;
-    }
-  }
-  // Loads are unconditional (see the streaming kernel): rows and tiles beyond the matrix are clamped, and
-  // k-tiles beyond the slice bring zero weights.
-  const bf16_t* xsrc[XJ];        // this lane's place in the activations at k-tile 0, for the token tiles it stages
-#pragma unroll
-  for (int j = 0; j < XJ; ++j) {
-    if constexpr (XF) xsrc[j] = x + ((size_t)min((m0 >> 4) + XJ * wave + j, (M - 1) >> 4) * KT * 64 + lane) * 8;
-    else xsrc[j] = x + (size_t)min(m0 + (XJ * wave + j) * 16 + r, M - 1) * K;
-  }
-  const bf16_t* wsrc[WN];
-#pragma unroll
-  for (int i = 0; i < WN; ++i) wsrc[i] = wf + (size_t)min(tile[i], NT - 1) * KT * 512 + lane * 8;
-
-  f32x4 acc[WN][TM];
-#pragma unroll
-  for (int i = 0; i < WN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  u32x4 xr[KC][XJ], wk[KC][WN];
-  const int kt_base = blockIdx.y * kt_per_slice, kt_end = min(KT, kt_base + kt_per_slice);
-  auto stage_load = [&](int s) {
-#pragma unroll
-    for (int kc = 0; kc < KC; ++kc)
-#pragma unroll
-      for (int j = 0; j < XJ; ++j) {
-        const int kt = max(0, min(kt_base + s * KC + kc, kt_end - 1));      // past the slice: the weights are zeros
-        if constexpr (XF) xr[kc][j] = *reinterpret_cast<const u32x4*>(xsrc[j] + (size_t)kt * 512);
-        else xr[kc][j] = *reinterpret_cast<const u32x4*>(xsrc[j] + min(kt * 32 + g * 8, K - 8));
-      }
-  };
-  auto stage_store = [&](int buf) {
-#pragma unroll
-    for (int kc = 0; kc < KC; ++kc)
-#pragma unroll
-      for (int j = 0; j < XJ; ++j) xs[((buf * KC + kc) * TM + XJ * wave + j) * 64 + lane] = xr[kc][j];
-  };
-  const bf16_t* zero = reinterpret_cast<const bf16_t*>(g_zero_tile) + lane * 8;
-  auto w_load = [&](int rel, u32x4 (&w)[WN]) {                // rel: k-tile relative to the slice
-    const int kt = kt_base + rel;
-    const bool kok = kt < kt_end;
-#pragma unroll
-    for (int i = 0; i < WN; ++i) w[i] = *reinterpret_cast<const u32x4*>(kok ? wsrc[i] + (size_t)kt * 512 : zero);
-  };
-  // blockIdx.y: the slice of the inner dimension this block sums (its own partial result y[slice][M][N])
-  const int kt_lo = blockIdx.y * kt_per_slice, kt_hi = min(KT, kt_lo + kt_per_slice);
-  const int S = (kt_hi - kt_lo + KC - 1) / KC;
-  y += (size_t)blockIdx.y * M * N;
-  stage_load(0);
-  stage_store(0);
-#pragma unroll
-  for (int kc = 0; kc < KC; ++kc) {
-    w_load(kc, wk[kc]);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  // Loads run one stage ahead and are unconditional (a k-tile beyond the slice in the last, partial stage
-  // reads the zero tile); the scheduling barriers keep them where they are issued, so that each wait is for
-  // the oldest loads only.
-  auto stage_mfma = [&](int s, bool more) {
-    u32x4 xf[TM];
-#pragma unroll
-    for (int j = 0; j < TM; ++j) xf[j] = xs[(((s & 1) * KC) * TM + j) * 64 + lane];
-#pragma unroll
-    for (int kc = 0; kc < KC; ++kc) {
-      const int kt_next = kt_base + (s + 1) * KC + kc;       // what this k-tile's weight registers hold next
-      const bool kok = kt_next < kt_end;
-#pragma unroll
-      for (int i = 0; i < WN; ++i) {
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          acc[i][j] = mfma16(wk[kc][i], xf[j], acc[i][j]);
-          // this token tile's fragment has had its last use: read the next k-tile's into the same registers
-          if (i == WN - 1 && kc + 1 < KC) xf[j] = xs[(((s & 1) * KC + kc + 1) * TM + j) * 64 + lane];
-        }
-        if (more) {
-          // this weight tile's registers are free again: fetch the same tile of the next stage now, so that the
-          // loads of a stage are spread over its products instead of arriving at the memory system in a burst
-          __builtin_amdgcn_sched_barrier(0);
-          wk[kc][i] = *reinterpret_cast<const u32x4*>(kok ? wsrc[i] + (size_t)kt_next * 512 : zero);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    }
-  };
-  for (int s = 0; s + 1 < S; ++s) {
-    stage_load(s + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
-    stage_mfma(s, true);
-    stage_store((s + 1) & 1);
-  }
-  if (S > 0) {                   // the last stage has nothing to fetch
-    __syncthreads();
-    stage_mfma(S - 1, false);
-  }
-
-  if constexpr (EPI == ALICE_EPI_ROPE) {
-    // The rotated values go to their places through LDS, 64 tokens at a time: a lane holds two pairs of a token
-    // (4-byte pieces of 16 different rows of q or of the cache), eight such stores per token tile and wave (measured:
-    // 4 to 6 % of the kernel against the staging below).  Staged, a token's 16 features of a weight tile become two runs of eight
-    // neighbouring elements of a head (the low and the high halves of eight pairs; a value head's 16 elements as
-    // they are), and every thread then moves 16-byte runs: along a token for q and for row-major caches, along 16
-    // tokens for keys in fragment order (a 1 KB tile per wave when the tokens start at a multiple of 16), and for
-    // values in fragment order eight tokens of one element at a time, which is that layout's 16-byte unit (when 32
-    // tokens are consecutive places of one sequence from a multiple of 32 on; one by one otherwise).
-    __shared__ RopeStagedToken tinfo[64];
-    __shared__ int group_ok[2];
-    bf16_t* stage = reinterpret_cast<bf16_t*>(xs_raw);
-    const int tid = threadIdx.x;
-    const int n_tile0 = bx * 4 * WN;
-    const int head0 = n_tile0 * 16 / ra.d;
-    const bool key_block = ra.layout == 1 && head0 >= ra.nH && head0 < ra.nH + ra.nKV;
-    const bool value_block = ra.layout == 1 && head0 >= ra.nH + ra.nKV;
-    // Every token's place first, then the cosines and sines one token tile ahead of their use: the loads of a
-    // tile are independent and in flight together.
-    RopeToken tk[TM];
-#pragma unroll
-    for (int j = 0; j < TM; ++j) tk[j] = rope_token(ra, min(m0 + j * 16 + r, M - 1));
-    RopeCol col[WN];
-#pragma unroll
-    for (int i = 0; i < WN; ++i) col[i] = rope_col(ra, min(tile[i], NT - 1) * 16 + g * 4);
-    RopeTrig tr[2][WN];
-    auto trig = [&](int j, RopeTrig (&o)[WN]) {
-#pragma unroll
-      for (int i = 0; i < WN; ++i) o[i] = rope_trig(ra, tk[j], col[i]);
-    };
-    trig(0, tr[0]);
-    auto emit = [&](int mb, int t, int c) {                  // run c (eight elements) of staged token t
-      const int nt = n_tile0 + (c >> 1);
-      const RopeStagedToken ti = tinfo[t];
-      if (nt >= NT || !ti.valid) return;
-      const int d = ra.d, head = nt * 16 / d, w0 = nt * 16 % d;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + t * ROPE_PITCH + c * 8);
-      if (head < ra.nH) {
-        const int dim0 = (w0 >> 1) + (c & 1) * (d >> 1);
-        *reinterpret_cast<u32x4*>(ra.q_out + ((size_t)(mb + t) * ra.nH + head) * d + dim0) = v;
-      } else if (!ti.page_ok) {
-        return;
-      } else if (head < ra.nH + ra.nKV) {
-        const int dim0 = (w0 >> 1) + (c & 1) * (d >> 1);
-        bf16_t* dst = ra.k_pool + ti.page_base + (size_t)(head - ra.nH) * ra.page_size * d;
-        *reinterpret_cast<u32x4*>(dst + k_offset(ra.layout, ti.tp, dim0, d)) = v;
-      } else {
-        const int dim0 = w0 + (c & 1) * 8;
-        bf16_t* dst = ra.v_pool + ti.page_base + (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
-        if (ra.layout == 0) {
-          *reinterpret_cast<u32x4*>(dst + (size_t)ti.tp * d + dim0) = v;
-        } else {
-          const bf16_t* e8 = stage + t * ROPE_PITCH + c * 8;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) dst[v_offset(1, ti.tp, dim0 + e, d)] = e8[e];
-        }
-      }
-    };
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      const int mb = m0 + (j & ~3) * 16;                     // the first of the 64 tokens being staged
-      if ((j & 3) == 0) {
-        __syncthreads();                                     // the memory's last readers are done
-        if (tid < 64) {
-          const int m = mb + tid, mc = min(m, M - 1), first = min(mb + (tid & 32), M - 1);
-          const RopeToken t = rope_token(ra, mc);
-          tinfo[tid] = RopeStagedToken{t.page_base, t.tp, m < M, t.page_ok};
-          const int pos0 = ra.positions[first];
-          const bool in_run = m < M && t.page_ok && ra.seq_of_token[mc] == ra.seq_of_token[first] &&
-                              t.pos == pos0 + (tid & 31) && (pos0 & 31) == 0 && (ra.page_size & 31) == 0;
-          const unsigned long long run = __ballot(in_run);
-          if (tid == 0) {
-            group_ok[0] = (run & 0xffffffffull) == 0xffffffffull;
-            group_ok[1] = (run >> 32) == 0xffffffffull;
-          }
-        }
-      }
-      if (j + 1 < TM) trig(j + 1, tr[(j + 1) & 1]);
-      uint32_t* row = reinterpret_cast<uint32_t*>(stage + ((j & 3) * 16 + r) * ROPE_PITCH + wave * (16 * WN));
-#pragma unroll
-      for (int i = 0; i < WN; ++i) {
-        float x[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[e] = round_to<bf16_t>(acc[i][j][e]);
-        if (col[i].head < ra.nH + ra.nKV) {
-          float l0, h0, l1, h1;
-          rotate_pair(x[0], x[1], tr[j & 1][i].c.x, tr[j & 1][i].s.x, l0, h0);
-          rotate_pair(x[2], x[3], tr[j & 1][i].c.y, tr[j & 1][i].s.y, l1, h1);
-          row[i * 8 + g] = pack_bf16x2(l0, l1);              // pairs 2 g and 2 g + 1 of the tile's eight: the low halves
-          row[i * 8 + 4 + g] = pack_bf16x2(h0, h1);          // and the high halves, eight elements on
-        } else {
-          row[i * 8 + 2 * g] = pack_bf16x2(x[0], x[1]);
-          row[i * 8 + 2 * g + 1] = pack_bf16x2(x[2], x[3]);
-        }
-      }
-      if ((j & 3) != 3) continue;
-      __syncthreads();
-      if (value_block) {
-        // wave items: (32 tokens, a 16-element tile of a head); a lane takes element lane % 16 of the tokens
-        // 4 (lane / 16) .. + 3 and the same 16 further on
-#pragma unroll 1
-        for (int it = 0; it < 8; ++it) {
-          const int item = it * 4 + wave, grp = item >> 4, vt = item & 15, nt = n_tile0 + vt;
-          if (nt >= NT) continue;
-          const int d = ra.d, head = nt * 16 / d, e = nt * 16 % d + (lane & 15), a = lane >> 4;
-          const bf16_t* src = stage + (grp * 32 + 4 * a) * ROPE_PITCH + vt * 16 + (lane & 15);
-          const size_t head_off = (size_t)(head - ra.nH - ra.nKV) * ra.page_size * d;
-          if (group_ok[grp]) {
-            uint16_t h[8];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              h[q] = src[q * ROPE_PITCH].bits;
-              h[4 + q] = src[(16 + q) * ROPE_PITCH].bits;
-            }
-            const u32x4 v = {h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16,
-                             h[6] | (uint32_t)h[7] << 16};
-            const RopeStagedToken ti = tinfo[grp * 32];
-            *reinterpret_cast<u32x4*>(ra.v_pool + ti.page_base + head_off + v_offset(1, ti.tp + 4 * a, e, d)) = v;
-          } else {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-              const int t = grp * 32 + 4 * a + (q & 3) + 16 * (q >> 2);
-              const RopeStagedToken ti = tinfo[t];
-              if (ti.valid && ti.page_ok)
-                ra.v_pool[ti.page_base + head_off + v_offset(1, ti.tp, e, d)] = src[((q & 3) + 16 * (q >> 2)) * ROPE_PITCH];
-            }
-          }
-        }
-      } else if (key_block) {
-        // wave items: (16 tokens, 32 elements of one half of a head); a lane takes run lane / 16 of token lane % 16
-#pragma unroll 1
-        for (int it = 0; it < 8; ++it) {
-          const int item = it * 4 + wave;
-          emit(mb, 16 * (item >> 3) + (lane & 15), 8 * ((item >> 1) & 3) + 2 * (lane >> 4) + (item & 1));
-        }
-      } else {
-#pragma unroll 2
-        for (int k = 0; k < 8; ++k) emit(mb, (tid >> 5) + 8 * k, tid & 31);
-      }
-    }
-    return;
-  }
-#pragma unroll
-  for (int j = 0; j < TM; ++j) {
-    const int m = m0 + j * 16 + r;
-    if (m >= M) continue;
-    const size_t row_off = (size_t)m * N;
-    if (EPI == ALICE_EPI_GEGLU) {
-#pragma unroll
-      for (int p = 0; p < WN / 2; ++p) {
-        if (tile[2 * p] >= NT) continue;
-        const int n = tile[2 * p] * 16 + g * 4;
-        f32x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
-        store4_any(y, y_frag, m, row_off, n, N, o);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < WN; ++i) {
-        if (tile[i] >= NT) continue;
-        const int n = tile[i] * 16 + g * 4;
-        f32x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = epilogue1<EPI, FULL>(acc[i][j][e], epi);
-        store4_any(y, y_frag, m, row_off, n, N, o);
-      }
-    }
-  }
+// What a tile costs at a few hundred tokens, in microseconds without the fixed part (fitted to all tiles and slice
+// counts at 96 to 1,024 tokens on the q|k|v, output, gate/up and down shapes of the 2B, 9B and 27B models; its
+// choices are 3 % behind the best measured one on average).  A block takes its k-tiles one after the other, each at
+// the slowest of: the wait for a stage's weights over the stage's k-tiles, the blocks' common share of the memory
+// rate, the bytes through the CU's L1, and the products; the busiest CU runs ceil(B / 256) blocks, two at a time.
+float tiled_cost(int M, int N, int K, int epi, int wn, int tm, int kc, int sp) {
+  const int NT = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16), KT = ceil_div(K, 32);
+  const int gx = ceil_div(NT, 4 * wn), gy = ceil_div(M, 16 * tm), B = gx * gy * sp, kts = ceil_div(KT, sp);
+  const int n = ceil_div(B, 256), res = n < 2 ? n : 2, conc = B < 512 ? B : 512;
+  float t = kc >= 8 ? 0.12f : kc >= 4 ? 0.146f : 0.25f;
+  t = fmaxf(t, (float)conc / gy * 4 * wn / 8000.f);
+  t = fmaxf(t, 0.011f * (4 * wn + tm) * res);
+  t = fmaxf(t, 0.008f * wn * tm * res);
+  const float rounds = n == 1 ? 1.f : (n / 2) + (n % 2) * 0.6f;
+  return rounds * kts * t + 0.1f * (sp > 1 ? sp : 0) * (float)M * N * 4e-6f;
 }
 
 template <int EPI, typename TO>
-int launch_tiled(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
-                 hipStream_t s, const RopeArgs& ra = RopeArgs{}) {
-  const int KT = (K + 31) / 32, NT = (N * (EPI == ALICE_EPI_GEGLU ? 2 : 1) + 15) / 16;
-  const int per = ceil_div(KT, split);
-  const int gx = EPI == ALICE_EPI_GEGLU ? ceil_div(N / 16, 4 * WN / 2) : ceil_div(NT, 4 * WN);
-  int gy = ceil_div(M, 16 * WM);
-  // 128 tokens a block, or 64 when that leaves most of the chip without a block (measured at N = 2304 and 4096:
-  // 216 and 256 blocks of 128 tokens beat twice as many of 64, 128 blocks do not; the same with the rotation
-  // epilogue since its stores go through LDS)
-  const bool high = gx * gy * split >= 192 || M <= 64;
-  if (!high) gy = ceil_div(M, 64);
-  dim3 grid(8 * ceil_div(gx * gy, 8), split);
-#define GO(TMV, XFV) \
-  linear_tiled_lds_kernel<EPI, TO, false, TMV, XFV><<<grid, 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w, (TO*)y, M, N, K, KT, NT, epi, gx, gy, per, y_frag, ra)
-  if (x_frag) { if (high) GO(8, true); else GO(4, true); }
-  else { if (high) GO(8, false); else GO(4, false); }
-#undef GO
-  ALICE_LAUNCH_CHECK();
-  return 0;
+int launch_wide(const void* x, const void* w, void* y, int M, int N, int K, int split, float epi, int x_frag, int y_frag,
+                hipStream_t s, int tm, const RopeArgs& ra) {
+  if (x_frag) {
+    if (tm == 8) return launch_tiled_as<EPI, TO, 8, true, 4, 2>(x, w, y, M, N, K, split, epi, y_frag, s, ra);
+    return launch_tiled_as<EPI, TO, 4, true, 4, 2>(x, w, y, M, N, K, split, epi, y_frag, s, ra);
+  }
+  if (tm == 8) return launch_tiled_as<EPI, TO, 8, false, 4, 2>(x, w, y, M, N, K, split, epi, y_frag, s, ra);
+  return launch_tiled_as<EPI, TO, 4, false, 4, 2>(x, w, y, M, N, K, split, epi, y_frag, s, ra);
+}
+
+bool narrow_built(int epi, int y_dtype) {
+  return (epi == ALICE_EPI_NONE && y_dtype == DT_F32) || (epi == ALICE_EPI_GEGLU && y_dtype == DT_BF16) || epi == ALICE_EPI_ROPE;
 }
 
 }  // namespace
 
+TiledPlan alice_mfma_tiled_plan(int M, int N, int K, int epi, int y_dtype, int split, int x_frag) {
+  const int KT = ceil_div(K, 32), NT = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
+  const bool may_split = epi == ALICE_EPI_NONE && y_dtype == DT_F32;
+  const int sp0 = split > 0 ? split : (may_split ? tiled_split_wide(M, N, K) : 1);
+  // The widest tile: 128 tokens a block, or 64 when that leaves most of the chip without a block (measured at
+  // N = 2304 and 4096: 216 and 256 blocks of 128 tokens beat twice as many of 64, 128 blocks do not; the same with
+  // the rotation epilogue since its stores go through LDS).
+  const bool high = ceil_div(NT, 16) * ceil_div(M, 128) * sp0 >= 192 || M <= 64;
+  const TiledPlan wide{4, high ? 8 : 4, 2, sp0};
+  // Between 65 and 1,024 tokens (what the cost rule was fitted on) another tile is taken where the rule says it is
+  // 8 % cheaper; the narrow tiles exist for activations in fragment order and for the layers' own products.
+  if (!(x_frag && M > 64 && M <= 1024 && narrow_built(epi, y_dtype))) return wide;
+  TiledPlan best = wide;
+  float best_cost = tiled_cost(M, N, K, epi, wide.wn, wide.tm, wide.kc, wide.split) * 0.92f;
+  static const int slices[] = {1, 2, 3, 4, 6, 8};
+  for (int wn = 4; wn >= 1; wn >>= 1) {
+    if (epi == ALICE_EPI_GEGLU && wn == 1) continue;
+    for (int tm = 8; tm >= 4; tm >>= 1) {
+      const int kc = wn == 4 ? 2 : 32 / tm;
+      for (int sp : slices) {
+        if (split > 0 ? sp != split : (sp > 1 && (!may_split || KT / sp < 16))) continue;
+        const float c = tiled_cost(M, N, K, epi, wn, tm, kc, sp);
+        if (c < best_cost) { best_cost = c; best = TiledPlan{wn, tm, kc, sp}; }
+      }
+    }
+  }
+  if (split > 0) best.split = split;
+  return best;
+}
+
 int alice_mfma_tiled(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K, int epi, float epi_param,
-                     int split, int x_frag, int y_frag, hipStream_t s) {
-  ALICE_MFMA_BY_EPI(launch_tiled, x, w, y, M, N, K, split, epi_param, x_frag, y_frag, s, RopeArgs{});
+                     int split, int x_frag, int y_frag, int force_wn, hipStream_t s) {
+  TiledPlan p = alice_mfma_tiled_plan(M, N, K, epi, y_dtype, split, x_frag);
+  p.split = split;
+  if (force_wn) {
+    ALICE_CHECK((force_wn == 1 || force_wn == 2) && x_frag && narrow_built(epi, y_dtype) && !(epi == ALICE_EPI_GEGLU && force_wn == 1),
+                "linear: no tiled kernel with a wave tile of %d features for this epilogue, output type and activation layout", 16 * force_wn);
+    p.wn = force_wn;
+    p.kc = 32 / p.tm;
+  }
+  if (p.wn < 4) return alice_mfma_tiled_narrow(x, w, y, y_dtype, M, N, K, epi, epi_param, p, y_frag, s, RopeArgs{});
+  const int tm = p.tm;
+  ALICE_MFMA_BY_EPI(launch_wide, x, w, y, M, N, K, split, epi_param, x_frag, y_frag, s, tm, RopeArgs{});
 }
 
 int alice_mfma_tiled_rope(const void* x, const void* w, int M, int N, int K, int x_frag, hipStream_t s, const RopeArgs& ra) {
-  return launch_tiled<ALICE_EPI_ROPE, bf16_t>(x, w, nullptr, M, N, K, 1, 0.f, x_frag, 0, s, ra);
+  const TiledPlan p = alice_mfma_tiled_plan(M, N, K, ALICE_EPI_ROPE, DT_BF16, 1, x_frag);
+  if (p.wn < 4) return alice_mfma_tiled_narrow(x, w, nullptr, DT_BF16, M, N, K, ALICE_EPI_ROPE, 0.f, p, 0, s, ra);
+  return launch_wide<ALICE_EPI_ROPE, bf16_t>(x, w, nullptr, M, N, K, 1, 0.f, x_frag, 0, s, p.tm, ra);
 }

@@ -17,7 +17,7 @@ from ..csrc import build as _build
 
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
-LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA = 0, 1, 2, 3
+LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
 ABI_VERSION = 4
 
 _lib = None
@@ -134,7 +134,9 @@ def _call(name: str, *args) -> None:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    # torch's current stream of the current device, as the raw handle: the same value as
+    # torch.cuda.current_stream().cuda_stream without building a Stream object for every launch
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def dtype_code(dt: torch.dtype) -> int:

@@ -570,6 +570,54 @@ def test_linear_mfma_geglu_in_fragment_order(M, N, K):
     assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 304, 160), (128, 2304, 2048), (200, 1000, 416), (257, 80, 1184), (700, 130, 96)])
+def test_linear_tiled_with_narrow_wave_tiles(M, N, K):
+    """The tiled kernel's wave tiles of 16 and 32 output features (prompts of a few hundred tokens), forced whatever
+    the cost rule would pick: float32 sums whole and in slices of the inner dimension, and the GeGLU epilogue, with
+    token counts that end inside a block, tile counts that a block's four waves do not divide, and inner dimensions
+    that are no multiple of a stage."""
+    x, w = rnd(M, K, seed=90, dtype=torch.bfloat16), rnd(N, K, seed=91, scale=0.1, dtype=torch.bfloat16)
+    wf, xf = ops.to_frag16(w), acts_to_fragments(x)
+    ref = x.double() @ w.double().T
+    wide = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(x, wf, wide, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_MFMA, full_precision=False)
+    for variant in (ops.LINEAR_TILED_W16, ops.LINEAR_TILED_W32):
+        for split in (1, 2, 3):
+            if split > 1 and K // 32 < 2 * split:
+                continue
+            y = torch.full((split, M, N) if split > 1 else (M, N), float("nan"), dtype=torch.float32, device=DEV)
+            ops.linear(xf, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=variant, full_precision=False,
+                       rows=M, x_layout=ops.LAYOUT_FRAG16)
+            if split == 1:
+                assert torch.equal(y, wide)                  # the same products in the same order
+            else:
+                close(y.sum(0), ref, 2e-4 * math.sqrt(K / 64), 1e-5)
+    if N % 16 == 0:
+        w2 = rnd(2 * N, K, seed=92, scale=0.3, dtype=torch.bfloat16)
+        gate, up = x.double() @ w2.double()[:N].T, x.double() @ w2.double()[N:].T
+        for y_layout in (ops.LAYOUT_ROW,) + ((ops.LAYOUT_FRAG16,) if N % 32 == 0 else ()):
+            frag = y_layout == ops.LAYOUT_FRAG16
+            yg = torch.full(((-(-M // 16) * 16) * N,) if frag else (M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ops.linear(xf, ops.to_frag16(w2), yg, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, epilogue=ops.EPI_GEGLU,
+                       variant=ops.LINEAR_TILED_W32, full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16, y_layout=y_layout)
+            got = acts_from_fragments(yg, M, N).to(DEV) if frag else yg
+            close(got, F.gelu(gate, approximate="tanh") * up, 2e-2 * math.sqrt(K / 64), 2 ** -7)
+    # what has no narrow kernel says so
+    y = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    with pytest.raises(ops.HipLibraryError, match="wave tile"):
+        ops.linear(x, wf, y, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=ops.LINEAR_TILED_W16, full_precision=False)
+
+
+def test_tiled_plan_splits_within_the_inner_dimension():
+    """The number of slices that the rule proposes for prompts keeps at least 16 k-tiles a slice and is one for
+    matrices that fill the chip by themselves."""
+    for M in (65, 128, 300, 512, 1024, 2048, 5000):
+        for N, K in ((2304, 2048), (2304, 9216), (4608, 36864), (18432, 2304), (64, 96), (3584, 512)):
+            s = ops.linear_split_hint(M, N, K, ops.LAYOUT_FRAG16)
+            assert 1 <= s <= 8 and (s == 1 or (K // 32) // s >= 16), (M, N, K, s)
+    assert ops.linear_split_hint(4096, 18432, 2304, ops.LAYOUT_FRAG16) == 1
+
+
 def test_linear_refuses_fragment_order_it_cannot_take():
     x, w = rnd(8, 40, seed=1, dtype=torch.bfloat16), rnd(48, 40, seed=2, dtype=torch.bfloat16)
     y = torch.empty(8, 48, dtype=torch.bfloat16, device=DEV)
