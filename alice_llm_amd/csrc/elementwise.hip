@@ -231,8 +231,9 @@ __global__ void add_norm_regs_kernel(float* __restrict__ resid, const float* __r
 }
 
 // The same operation for many rows (prompts): one wave per row, four rows a block, four consecutive
-// elements a lane at a time (H a multiple of 4, at most 256 * K4).  No barriers: the sums go through the
-// wave's lanes.  Reduction orders differ from the block-per-row kernels by rounding only.
+// elements a lane at a time (H a multiple of 4, at most 256 * K4); or, for rows too wide for one wave's
+// registers, two waves per row (WPR = 2, at most 512 * K4 elements: the first wave takes the first 256 * K4),
+// whose sums meet in LDS.  Reduction orders differ from the block-per-row kernels by rounding only.
 template <typename TW> __device__ __forceinline__ float4 load4_f32(const TW* p, int e);
 template <> __device__ __forceinline__ float4 load4_f32<float>(const float* p, int e) { return *reinterpret_cast<const float4*>(p + e); }
 template <> __device__ __forceinline__ float4 load4_f32<bf16_t>(const bf16_t* p, int e) {
@@ -240,24 +241,38 @@ template <> __device__ __forceinline__ float4 load4_f32<bf16_t>(const bf16_t* p,
   return float4{bf16_bits_to_f32(v.x & 0xffffu), bf16_bits_to_f32(v.x >> 16), bf16_bits_to_f32(v.y & 0xffffu), bf16_bits_to_f32(v.y >> 16)};
 }
 
-template <typename TW, typename TO, bool FULL, int K4>
+template <typename TW, typename TO, bool FULL, int K4, int WPR>
 __global__ __launch_bounds__(256) void add_norm_rows_kernel(float* __restrict__ resid, const float* __restrict__ branch,
                                                             int n_partials, size_t partial_stride,
                                                             const TW* __restrict__ w_post, const TW* __restrict__ w_pre,
                                                             TO* __restrict__ out, int T, int H,
                                                             float eps_post, float eps_pre, float off_post, float off_pre,
                                                             int out_layout) {
-  const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= T) return;
+  __shared__ float red[2][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, part = wave % WPR;
+  const int r_own = blockIdx.x * (4 / WPR) + wave / WPR;
+  if (WPR == 1 && r_own >= T) return;
+  const bool row_ok = r_own < T;                              // two waves a row: every wave reaches the barriers
+  const int r = row_ok ? r_own : T - 1;
   const size_t src = (size_t)r * H;
   int e[K4];
   bool ok[K4];
 #pragma unroll
   for (int k = 0; k < K4; ++k) {
-    const int i = (k * 64 + lane) * 4;
-    ok[k] = i < H;
+    const int i = ((part * K4 + k) * 64 + lane) * 4;
+    ok[k] = i < H && row_ok;
     e[k] = min(i, H - 4);                                    // clamped: loads are unconditional
   }
+  // the row's sum of squares from its waves' shares, the same addends in the same order in both
+  auto row_sum = [&](float ss, int which) {
+    ss = wave_sum(ss);
+    if constexpr (WPR == 2) {
+      if (lane == 0) red[which][wave] = ss;
+      __syncthreads();
+      ss = red[which][wave & ~1] + red[which][wave | 1];
+    }
+    return ss;
+  };
   const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
   float4 xv[K4], bv[K4];
 #pragma unroll
@@ -282,7 +297,7 @@ __global__ __launch_bounds__(256) void add_norm_rows_kernel(float* __restrict__ 
       float ss = 0.f;
 #pragma unroll
       for (int k = 0; k < K4; ++k) ss += bv[k].x * bv[k].x + bv[k].y * bv[k].y + bv[k].z * bv[k].z + bv[k].w * bv[k].w;
-      ss = wave_sum(ss);
+      ss = row_sum(ss, 0);
       const float mean = ss / (float)H;
       const float inv_b = FULL ? 1.f / sqrtf(mean + eps_post) : rsqrtf(mean + eps_post);
 #pragma unroll
@@ -306,7 +321,7 @@ __global__ __launch_bounds__(256) void add_norm_rows_kernel(float* __restrict__ 
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < K4; ++k) ss += xv[k].x * xv[k].x + xv[k].y * xv[k].y + xv[k].z * xv[k].z + xv[k].w * xv[k].w;
-    ss = wave_sum(ss);
+    ss = row_sum(ss, 1);
     const float mean = ss / (float)H;
     inv = FULL ? 1.f / sqrtf(mean + eps_pre) : rsqrtf(mean + eps_pre);
   }
@@ -349,17 +364,21 @@ extern "C" int alice_add_norm(float* resid, const float* branch, int n_partials,
   }
 #define ARGS resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, rows, H, \
              eps_post, eps_pre, off_post, off_pre, out_layout
-  // Many rows, no gather: a wave per row.
+  // Many rows, no gather: a wave per row (two from 4,097 elements on).  From 320 rows: below, a block per row
+  // fills more of the chip (measured at 2,304 and 3,584 elements: up to 256 rows the block-per-row kernel is 0.5
+  // to 6 us faster, from 384 rows on the wave-per-row kernel is, by half at 2,048 rows).
   const bool aligned = (((uintptr_t)resid | (uintptr_t)branch | (uintptr_t)out | (uintptr_t)w_post | (uintptr_t)w_pre) & 15) == 0;
-  const int k4 = (!rows && aligned && T >= 128 && H % 4 == 0 && H >= 256 && H <= 4096 && (partial_stride % 4 == 0 || !branch)) ? ceil_div(H, 256) : 0;
-#define ROWS(TW, TO, FULL, K4) add_norm_rows_kernel<TW, TO, FULL, K4><<<ceil_div(T, 4), 256, 0, stream>>>(                \
+  const int k4 = (!rows && aligned && T >= 320 && H % 4 == 0 && H >= 256 && H <= 8192 && (partial_stride % 4 == 0 || !branch)) ? ceil_div(H, 256) : 0;
+#define ROWS(TW, TO, FULL, K4, WPR) add_norm_rows_kernel<TW, TO, FULL, K4, WPR><<<ceil_div(T, 4 / WPR), 256, 0, stream>>>(     \
     resid, branch, n_partials, (size_t)partial_stride, (const TW*)w_post, (const TW*)w_pre, (TO*)out, T, H, eps_post, eps_pre, \
     off_post, off_pre, out_layout)
 #define LAUNCH(TW, TO, FULL)                                                                         \
   do {                                                                                               \
-    if (k4 > 0 && k4 <= 4) ROWS(TW, TO, FULL, 4);                                                    \
-    else if (k4 > 4 && k4 <= 9) ROWS(TW, TO, FULL, 9);                                               \
-    else if (k4 > 9) ROWS(TW, TO, FULL, 16);                                                         \
+    if (k4 > 0 && k4 <= 4) ROWS(TW, TO, FULL, 4, 1);                                                 \
+    else if (k4 > 4 && k4 <= 9) ROWS(TW, TO, FULL, 9, 1);                                            \
+    else if (k4 > 9 && k4 <= 16) ROWS(TW, TO, FULL, 16, 1);                                          \
+    else if (k4 > 16 && k4 <= 18) ROWS(TW, TO, FULL, 9, 2);                                          \
+    else if (k4 > 18) ROWS(TW, TO, FULL, 16, 2);                                                     \
     else if (ept == 1) add_norm_regs_kernel<TW, TO, FULL, 1><<<T, threads, 0, stream>>>(ARGS);            \
     else if (ept == 2) add_norm_regs_kernel<TW, TO, FULL, 2><<<T, threads, 0, stream>>>(ARGS);       \
     else if (ept == 4) add_norm_regs_kernel<TW, TO, FULL, 4><<<T, threads, 0, stream>>>(ARGS);       \

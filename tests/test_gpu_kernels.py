@@ -70,12 +70,13 @@ def test_add_norm_all_forms(wdt, odt, full, H):
     close(out3, P.rms_norm(x0.double()[rows.long()], wq.double(), 1e-5), tol, tol)
 
 
-@pytest.mark.parametrize("H", [256, 1000, 2304, 4096])
+@pytest.mark.parametrize("H", [256, 1000, 2304, 4096, 4608, 5000, 8192])
 @pytest.mark.parametrize("S", [1, 3])
 @pytest.mark.parametrize("odt", ["float32", "bfloat16"])
 def test_add_norm_many_rows(H, S, odt):
-    # prompts take another kernel (a wave per row) than single tokens do
-    T = 300
+    # long prompts take another kernel (a wave per row, two waves from 4,097 elements on) than single tokens do;
+    # the last block has a row too few
+    T = 333
     x0 = rnd(T, H, seed=2, scale=3.0)
     br = rnd(S, T, H, seed=3, scale=0.5) if S > 1 else rnd(T, H, seed=3, scale=0.5)
     wp, wq = rnd(H, seed=4, scale=0.1, dtype=torch.bfloat16), rnd(H, seed=5, scale=0.1, dtype=torch.bfloat16)
