@@ -12,6 +12,8 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence
 
+import torch
+
 
 @dataclass
 class GenerationResult:
@@ -103,6 +105,13 @@ class Generator:
         return results  # type: ignore[return-value]
 
     def _run_batch(self, batch, prompts, caps, results) -> None:
+        """One batch from its prompts to its last token.  With an engine that takes token ids as a device tensor
+        (and no observer to show every step to), the loop runs one step ahead of what it has seen: step n + 1 is
+        queued, fed from the sampling kernel's output on the device, before the ids of step n have reached the
+        host, so the GPU does not wait for the host between two steps.  Ends by a cap are known beforehand; a
+        sequence that draws a stop token has by then been queued for one more step, whose result is dropped (its
+        slot is given back at once: the pages it may hand to a later step are written by that step after this
+        one)."""
         eng = self.engine
         out = {r: [] for r in batch}
         reason = {}
@@ -111,21 +120,39 @@ class Generator:
             if caps[r] <= 0:
                 reason[r] = "length"
         slots = dict(zip(live, eng.open(len(live))))
+        ahead = self.observer is None and getattr(eng, "takes_device_tokens", False)
         t0 = time.perf_counter()
         prefill_ms = 0.0
         try:
-            feed = [list(prompts[r]) for r in live]
+            rows = list(live)                                # the requests of the step whose ids are on their way
+            drawn = None                                     # that step's ids on the device and, later, on the host
+            if rows:
+                logits = eng.step([slots[r] for r in rows], [list(prompts[r]) for r in rows], "last")
+                drawn = self._draw(logits, rows, out, 0)
             first = True
-            while live:
-                logits = eng.step([slots[r] for r in live], feed, "last")
-                ids = self.sampler(logits, live, [len(out[r]) for r in live]).tolist()   # waits for the step
-                if self.observer is not None:
-                    self.observer(list(live), [len(prompts[r]) + len(out[r]) - 1 for r in live], logits, ids)
+            while rows:
+                queued = None
+                alive = [r for r in rows if r not in reason]
+                if ahead:
+                    # the sequences that go on unless they draw a stop token now
+                    nxt = [r for r in alive if len(out[r]) + 1 < caps[r]]
+                    if nxt:
+                        ids_dev = drawn[0]
+                        if len(nxt) != len(rows):
+                            pick = torch.tensor([rows.index(r) for r in nxt], dtype=torch.int64)
+                            ids_dev = ids_dev[pick.to(ids_dev.device)]
+                        logits = eng.step([slots[r] for r in nxt], ids_dev, "last")
+                        queued = (nxt, self._draw(logits, nxt, out, 1))
+                ids = drawn[1]()                             # waits for the step before the queued one only
                 if first:
                     prefill_ms = (time.perf_counter() - t0) * 1e3
                     first = False
-                still, feed = [], []
-                for r, tok in zip(live, ids):
+                if self.observer is not None:
+                    self.observer(list(rows), [len(prompts[r]) + len(out[r]) - 1 for r in rows], drawn[2], ids)
+                feed = []
+                for r, tok in zip(rows, ids):
+                    if r in reason:                          # ended a step ago: this row ran ahead for nothing
+                        continue
                     tok = int(tok)
                     if tok in self.stop:
                         if self.include_stop_token:
@@ -138,9 +165,17 @@ class Generator:
                     if r in reason:
                         eng.close([slots.pop(r)])            # the slot is free for the next batch at once
                     else:
-                        still.append(r)
-                        feed.append([tok])
-                live = still
+                        feed.append((r, tok))
+                if queued is not None:
+                    rows, drawn = queued
+                    if all(r in reason for r in rows):
+                        rows = []
+                elif feed:
+                    rows = [r for r, _ in feed]
+                    logits = eng.step([slots[r] for r in rows], [[tok] for _, tok in feed], "last")
+                    drawn = self._draw(logits, rows, out, 0)
+                else:
+                    rows = []
         finally:
             if slots:
                 eng.close(list(slots.values()))
@@ -148,3 +183,19 @@ class Generator:
         for r in batch:
             results[r] = GenerationResult(tokens=out[r], finish_reason=reason[r], prompt_tokens=len(prompts[r]),
                                           prefill_ms=prefill_ms, decode_ms=decode_ms)
+
+    def _draw(self, logits, rows, out, pending: int):
+        """Samples a step's rows (request r has drawn len(out[r]) + pending tokens before).  Returns the ids on
+        the device, a function that gives them as a list once they have reached the host, and the logits."""
+        ids = self.sampler(logits, rows, [len(out[r]) + pending for r in rows])
+        if not (isinstance(ids, torch.Tensor) and ids.is_cuda):
+            return ids, ids.tolist, logits
+        host = torch.empty(ids.shape, dtype=ids.dtype, pin_memory=True)
+        host.copy_(ids, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+
+        def fetch():
+            done.synchronize()
+            return host.tolist()
+        return ids, fetch, logits

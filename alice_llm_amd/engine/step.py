@@ -166,6 +166,8 @@ class _DecodeGraph:
 class Engine:
     """A model, its cache, and the step function over them."""
 
+    takes_device_tokens = True      # step() accepts one token id per sequence as a device tensor
+
     def __init__(self, model: CausalLM, *, max_tokens: Optional[int] = None, seq_lens: Optional[Sequence[int]] = None,
                  max_seqs: Optional[int] = None, use_graphs: Optional[bool] = None, max_graphs: int = 24,
                  page_size: int = PAGE_SIZE):
@@ -209,13 +211,24 @@ class Engine:
         return self.cache.page_size
 
     # ------------------------------------------------------------------ the step
-    def step(self, slots: Sequence[int], new_tokens: Sequence[Sequence[int]], want: Want = "last") -> torch.Tensor:
+    def step(self, slots: Sequence[int], new_tokens, want: Want = "last") -> torch.Tensor:
         """Run new_tokens[i] for the sequence in slots[i]; returns float32 logits [n_wanted, vocab].
 
+        new_tokens: per sequence the list of its next token ids; or, for one token each, an int32 tensor [B] on
+        the engine's device (what the sampling kernels return): the step is then queued without the host ever
+        seeing the ids, so that a loop can queue the next step while this one runs.  An id outside the
+        vocabulary, which the host cannot refuse then, embeds as a row of zeros.
         want: "last" (the last new token of each sequence), "all", "none", or per sequence a list of
         indices into its new tokens.  Rows come in the order of the sequences and of their lists.
         """
         B = len(slots)
+        device_tokens = None
+        if isinstance(new_tokens, torch.Tensor):
+            if (new_tokens.dtype != torch.int32 or new_tokens.device != self.device or new_tokens.dim() != 1
+                    or not new_tokens.is_contiguous()):
+                raise ValueError(f"token ids given as a tensor must be contiguous int32 [sequences] on {self.device}")
+            device_tokens = new_tokens
+            new_tokens = [[0]] * new_tokens.numel()
         if B == 0 or len(new_tokens) != B:
             raise ValueError("a step needs at least one sequence and one token list per sequence")
         n_new = [len(t) for t in new_tokens]
@@ -243,7 +256,7 @@ class Engine:
         self.cache.reserve(slots, n_new)                       # raises before any launch
 
         if self.use_graphs and want == "last" and max(n_new) == 1:
-            logits = self._graph_step(slots, flat, start)
+            logits = self._graph_step(slots, flat, start, device_tokens)
             self.cache.commit(slots, n_new)
             return logits
 
@@ -266,6 +279,8 @@ class Engine:
             offs.append(offs[-1] + len(p))
         part = lambda i: packed[offs[i]:offs[i + 1]]
         block_tables = [part(7 + g).view(B, width) for g in range(len(tables))]
+        if device_tokens is not None:
+            part(0).copy_(device_tokens)
         ctx = StepContext(tokens=part(0), positions=part(1), seq_of_token=part(2), slots=part(3),
                           want_rows=part(4) if rows else None, cu_seqlens=part(5), context_lens=part(6),
                           n_tokens=T, n_seqs=B, is_decode=all(n == 1 for n in n_new), max_new=max(n_new),
@@ -278,7 +293,7 @@ class Engine:
         return logits
 
     # ------------------------------------------------------------------ captured decode steps
-    def _graph_step(self, slots, tokens, start) -> torch.Tensor:
+    def _graph_step(self, slots, tokens, start, device_tokens=None) -> torch.Tensor:
         """One token per sequence through a captured HIP graph.  The batch is padded to a bucket size with
         rows that read and write only the cache's spare page; their logits are dropped."""
         B = len(slots)
@@ -292,6 +307,8 @@ class Engine:
         else:
             self._graphs[key] = self._graphs.pop(key)          # most recently used last
         g.fill(self, slots, tokens, start)
+        if device_tokens is not None:
+            g.ctx.tokens[:B].copy_(device_tokens)            # after the queued copy of the step's other integers
         if g.graph is None:
             # The first step of a bucket runs eagerly (which also warms up whatever the capture must not do for
             # the first time) and is then recorded without being run again: a part with state of its own would

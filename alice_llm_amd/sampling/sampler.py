@@ -8,7 +8,7 @@ request's tokens do not depend on which other requests share its batch.
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -41,6 +41,11 @@ class Sampler:
         if not top_p > 0:
             raise ValueError("top_p must be positive (1 turns it off)")
         self.temperature, self.top_k, self.top_p, self.seed = float(temperature), int(top_k), float(top_p), int(seed)
+        # pinned host buffers for the uniform numbers, used in turn: their copies are queued behind the step's
+        # kernels without the host waiting for them (a copy from ordinary memory would wait)
+        self._pinned: List[Optional[torch.Tensor]] = [None] * 4
+        self._copied: List[Optional[torch.cuda.Event]] = [None] * 4
+        self._turn = 0
 
     @property
     def greedy(self) -> bool:
@@ -52,4 +57,18 @@ class Sampler:
         if self.greedy:
             return ops.argmax(logits)
         u = torch.tensor([uniform(self.seed, r, n) for r, n in zip(requests, draws)], dtype=torch.float32)
-        return ops.sample(logits, u.to(logits.device), self.temperature, self.top_k, self.top_p)
+        return ops.sample(logits, self._upload(u, logits.device), self.temperature, self.top_k, self.top_p)
+
+    def _upload(self, u: torch.Tensor, device) -> torch.Tensor:
+        i = self._turn = (self._turn + 1) % len(self._pinned)
+        if self._copied[i] is not None:
+            self._copied[i].synchronize()                    # the copy that last read this buffer has run
+        if self._pinned[i] is None or self._pinned[i].numel() < u.numel():
+            self._pinned[i] = torch.empty(max(64, 2 * u.numel()), dtype=torch.float32).pin_memory()
+        host = self._pinned[i][:u.numel()]
+        host.copy_(u)
+        out = torch.empty(u.numel(), dtype=torch.float32, device=device)
+        out.copy_(host, non_blocking=True)
+        self._copied[i] = torch.cuda.Event()
+        self._copied[i].record()
+        return out

@@ -80,6 +80,8 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure decode at ('' for none)")
     ap.add_argument("--point-steps", type=int, default=None, help="steps for the other batch sizes (default: --steps)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--ids-through-host", action="store_true",
+                    help="read every step's chosen ids on the host before the next step is queued (the loop with an observer)")
     ap.add_argument("--prefill-tokens", default="2048,8192", help="prompt lengths whose prefill is timed (the first is the headline's)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -131,13 +133,36 @@ def main() -> int:
             ids += ops.argmax(logits).tolist()
             i = j
             print(f"[bench] prefilled {i}/{batch}", file=sys.stderr, flush=True)
+        # Decode steps as the library's own generation loop runs them: the chosen ids go from the sampling kernel
+        # to the next step on the device, and the host queues step n + 1 before it reads step n's ids (through a
+        # pinned buffer and an event), so it is one step ahead and no further.
+        pending = []
+
+        def one(ids):
+            if args.ids_through_host:
+                return ops.argmax(eng.step(slots, [[t_] for t_ in ids], "last")).tolist()
+            out = ops.argmax(eng.step(slots, ids, "last"))
+            host = torch.empty(out.shape, dtype=out.dtype, pin_memory=True)
+            host.copy_(out, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            pending.append((ev, host))
+            if len(pending) > 1:
+                ev0, host0 = pending.pop(0)
+                ev0.synchronize()
+                host0.tolist()                                   # where a loop would look for stop tokens
+            return out
+
+        if not args.ids_through_host:
+            ids = torch.tensor(ids, dtype=torch.int32, device="cuda")
         for _ in range(warmup):
-            ids = ops.argmax(eng.step(slots, [[t] for t in ids], "last")).tolist()
+            ids = one(ids)
         ctx0 = [eng.length(s) for s in slots]
         sync()
+        pending.clear()
         t = time.perf_counter()
         for _ in range(steps):
-            ids = ops.argmax(eng.step(slots, [[t_] for t_ in ids], "last")).tolist()
+            ids = one(ids)
         sync()
         dt = time.perf_counter() - t
         ctx1 = [eng.length(s) for s in slots]

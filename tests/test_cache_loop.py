@@ -226,6 +226,51 @@ def test_loop_stop_tokens_caps_and_slot_reuse():
     assert gen2.run([[7]], [10])[0].tokens == [8, 9]
 
 
+class FakeEngineAhead(FakeEngine):
+    """The same, and it takes one token id per sequence as a tensor, as the GPU engine does: the loop then
+    queues a step before it has seen the ids of the step before."""
+    takes_device_tokens = True
+
+    def step(self, slots, tokens, want):
+        if isinstance(tokens, torch.Tensor):
+            assert tokens.dim() == 1 and tokens.numel() == len(slots)
+            self.from_tensor = getattr(self, "from_tensor", 0) + 1
+            tokens = [[int(t)] for t in tokens]
+        return super().step(slots, tokens, want)
+
+
+def test_loop_one_step_ahead_decides_as_the_plain_loop_does():
+    prompts = [[1, 2, 3], [7], [4, 5], [12, 13, 14, 15], [2], [6], [5]]
+    caps = [4, 10, 0, 3, 2, 1, 9]
+    runs = []
+    for cls in (FakeEngine, FakeEngineAhead):
+        eng = cls(n_slots=4)
+        gen = Generator(eng, stop_token_ids=[9], max_batch=3, sampler=argmax_sampler)
+        res = gen.run(prompts, caps)
+        runs.append(([r.tokens for r in res], [r.finish_reason for r in res]))
+        assert sorted(eng.opened) == sorted(eng.closed)                 # every slot given back, once
+        assert len(set(eng.opened)) <= 3
+        eng.cache.check_consistent()
+        assert eng.cache.slots.n_free() == 4
+    assert runs[0] == runs[1]
+    assert runs[1][0] == [[4, 5, 6, 7], [8], [], [0, 1, 2], [3, 4], [7], [6, 7, 8]]
+    assert runs[1][1] == ["length", "stop", "length", "length", "length", "length", "stop"]
+    assert eng.from_tensor > 0
+    # Request 1 draws the stop token 9 in its second step; by then the loop had queued it for a third, whose row is
+    # dropped: one row more than the plain loop ran, in that step only.  Ends by a cap are never run past.
+    plain, ahead = FakeEngine(n_slots=4), FakeEngineAhead(n_slots=4)
+    for eng in (plain, ahead):
+        Generator(eng, stop_token_ids=[9], sampler=argmax_sampler).run([[1, 2, 3], [7]], [4, 10])
+    assert [len(s) for s, _ in plain.steps] == [2, 2, 1, 1]
+    assert [len(s) for s, _ in ahead.steps] == [2, 2, 2, 1]
+    # an observer sees every step as it is: the loop then waits for each
+    seen = []
+    eng = FakeEngineAhead()
+    Generator(eng, stop_token_ids=[9], sampler=argmax_sampler,
+              observer=lambda requests, positions, logits, tokens: seen.append(list(tokens))).run([[1, 2, 3], [7]], [3, 5])
+    assert seen == [[4, 8], [5, 9], [6]] and not hasattr(eng, "from_tensor")
+
+
 def test_loop_gives_slots_back_on_error():
     eng = FakeEngine(max_tokens=128)
     def bad_sampler(logits, requests, draws):

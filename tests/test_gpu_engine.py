@@ -204,6 +204,46 @@ def test_captured_decode_steps_match_eager_on_every_replay(name, dtype):
     graph.cache.check_consistent()
 
 
+@pytest.mark.parametrize("name,dtype", [("tiny-c", "bfloat16"), ("tiny-b", "float32")])
+@pytest.mark.parametrize("graphs", [True, False])
+def test_token_ids_given_on_the_device(name, dtype, graphs):
+    """One token id per sequence as a device tensor (what the sampling kernels return) gives the same bits as the
+    same ids from the host, in captured and in eager steps, fed from the step before without the host seeing
+    them; a batch that shrinks takes the ids of the rows that go on."""
+    model, plain = setup(name, dtype)
+    prompts = [random_tokens(plain.V, n, 70 + i) for i, n in enumerate((5, 40, 66))]
+    a = model.engine(max_tokens=64 * 12, max_seqs=4, use_graphs=graphs)
+    b = model.engine(max_tokens=64 * 12, max_seqs=4, use_graphs=graphs)
+    sa, sb = a.open(3), b.open(3)
+    ids_a = alice.sample(a.step(sa, prompts, "last"))
+    ids_b = alice.sample(b.step(sb, prompts, "last"))
+    assert torch.equal(ids_a, ids_b)
+    seqs = [list(p) for p in prompts]
+    for step in range(6):
+        host = ids_a.tolist()
+        for s, t in zip(seqs, host):
+            s.append(t)
+        la = a.step(sa, [[t] for t in host], "last")
+        lb = b.step(sb, ids_b, "last")                       # never read on the host
+        assert torch.equal(la, lb), step
+        ids_a, ids_b = alice.sample(la), alice.sample(lb)
+        if step == 2:                                        # the middle sequence ends
+            a.close([sa.pop(1)]); b.close([sb.pop(1)]); seqs.pop(1)
+            ids_a = ids_a[[0, 2]].contiguous()
+            ids_b = ids_b[torch.tensor([0, 2], device=ids_b.device)]
+    for s, la_row in zip(seqs, la):                          # and the ids were the greedy ones of the plain model
+        ref = plain.forward(s)[-1]
+        assert max_err(la_row, ref) < tol(dtype, ref)
+    with pytest.raises(ValueError):
+        b.step(sb, ids_b.long(), "last")
+    with pytest.raises(ValueError):
+        b.step(sb, ids_b.cpu(), "last")
+    # an id outside the vocabulary cannot be refused by the host then: it embeds as zeros, and nothing is read out of bounds
+    bad = torch.tensor([plain.V + 5, -1], dtype=torch.int32, device=ids_b.device)
+    assert torch.isfinite(b.step(sb, bad, "last")).all()
+    a.cache.check_consistent(); b.cache.check_consistent()
+
+
 @pytest.mark.parametrize("name,dtype", [("tiny-b", "float32"), ("tiny-c", "bfloat16"), ("tiny-c", "float32")])
 def test_stale_cache_contents_and_slot_order_change_nothing(name, dtype):
     """Pages are handed out again without being cleared.  Here every page of every pool is first filled with

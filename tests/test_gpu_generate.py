@@ -72,6 +72,32 @@ def test_temperature_sampling_is_reproducible_and_batch_independent():
     assert greedy == cold
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_loop_one_step_ahead_gives_what_the_waiting_loop_gives(dtype):
+    """Generation queues step n + 1 from the ids on the device before the host has seen step n's; with an observer
+    it waits for every step.  Both give the same tokens and reasons: with stop tokens drawn in the middle (the
+    sequence has by then run one step ahead, and its slot goes to the next batch), unequal caps, several batches
+    on few slots, greedy and with a temperature."""
+    folder = model_folder("tiny-b", "bfloat16")
+    plain = plain_model(folder)
+    prompts = [random_tokens(plain.V, n, 90 + i) for i, n in enumerate((3, 9, 14, 21, 2, 33, 7))]
+    model = alice.load(folder, dtype=dtype)
+    free = model.generate(prompts, max_new_tokens=12, stop_token_ids=[])
+    stops = [free[1].tokens[4], free[3].tokens[1], free[5].tokens[8]]
+    caps = [12, 9, 1, 12, 5, 12, 2]
+    seen = []
+    for kw in (dict(), dict(temperature=0.9, seed=5, top_k=20)):
+        runs = []
+        for observer in (None, lambda requests, positions, logits, tokens: seen.append(len(tokens))):
+            for max_batch in (None, 3):
+                res = model.generate(prompts, max_new_tokens=caps, stop_token_ids=stops, max_batch=max_batch, observer=observer, **kw)
+                runs.append([(r.tokens, r.finish_reason) for r in res])
+        assert all(r == runs[0] for r in runs[1:])
+        assert any(reason == "stop" for _, reason in runs[0]) and any(reason == "length" for _, reason in runs[0])
+        assert all(len(t) <= c and not set(t) & set(stops) for (t, _), c in zip(runs[0], caps))
+    assert seen
+
+
 def test_command_line(tmp_path):
     folder = model_folder("tiny-a", "bfloat16")
     plain = plain_model(folder)
