@@ -206,6 +206,7 @@ int alice_mfma_tiled(const void* x, const void* w, void* y, int y_dtype, int M, 
 int alice_mfma_tiled_rope(const void* x, const void* w, int M, int N, int K, int x_frag, hipStream_t s, const RopeArgs& ra);
 // The tiled kernel's tile: a wave's 16 wn output features x 16 tm tokens, kc k-tiles a stage, slices of the inner
 // dimension.  split 0: the rule chooses the slices too (float32 sums without epilogue only), else they are given.
+// Up to 64 tokens wn is 0 where the streaming kernel is the better one (always up to 32).
 struct TiledPlan { int wn, tm, kc, split; };
 TiledPlan alice_mfma_tiled_plan(int M, int N, int K, int epi, int y_dtype, int split, int x_frag);
 int alice_mfma_tiled_narrow(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K, int epi, float epi_param,

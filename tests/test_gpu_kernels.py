@@ -461,8 +461,29 @@ def test_linear_streaming_with_six_row_tiles(M):
     split = ops.linear_split_hint(M, N, K, ops.LAYOUT_FRAG16)
     assert split > 1
     yp = torch.full((split, M, N), float("nan"), dtype=torch.float32, device=DEV)
-    ops.linear(x, ops.to_frag16(w), yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False)
+    ops.linear(x, ops.to_frag16(w), yp, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=ops.LINEAR_SKINNY,
+               full_precision=False)
     close(yp.sum(0), x.double() @ w.double().T, 2e-4 * math.sqrt(K / 64), 1e-5)
+
+
+def test_between_33_and_64_tokens_the_rule_picks_a_kernel_and_both_agree():
+    """From 33 to 64 tokens with activations in fragment order the launcher takes the tiled kernel's narrow tiles where
+    their blocks come close to one a CU, the streaming kernel elsewhere; whichever it takes, the sums are those of
+    the streaming kernel up to rounding, and the number of slices it proposes is one it can run."""
+    for M, N, K in ((40, 2304, 9216), (64, 2304, 2048), (64, 4096, 2304), (33, 8192, 512), (50, 1024, 8192)):
+        x, w = rnd(M, K, seed=95, dtype=torch.bfloat16), rnd(N, K, seed=96, scale=0.1, dtype=torch.bfloat16)
+        wf, xf = ops.to_frag16(w), acts_to_fragments(x)
+        split = ops.linear_split_hint(M, N, K, ops.LAYOUT_FRAG16)
+        shape = (split, M, N) if split > 1 else (M, N)
+        a = torch.full(shape, float("nan"), dtype=torch.float32, device=DEV)
+        b = torch.full(shape, float("nan"), dtype=torch.float32, device=DEV)
+        ops.linear(xf, wf, a, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, full_precision=False, rows=M,
+                   x_layout=ops.LAYOUT_FRAG16)
+        ops.linear(xf, wf, b, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, split_k=split, variant=ops.LINEAR_SKINNY,
+                   full_precision=False, rows=M, x_layout=ops.LAYOUT_FRAG16)
+        ref = x.double() @ w.double().T
+        for y in (a, b):
+            close(y.sum(0) if split > 1 else y, ref, 2e-4 * math.sqrt(K / 64), 1e-5)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 9216, 128), (40, 416, 160), (64, 48, 96), (200, 304, 96), (129, 2048, 64)])
@@ -571,10 +592,11 @@ def test_linear_mfma_geglu_in_fragment_order(M, N, K):
     assert torch.equal(acts_from_fragments(yf, M, N), row.cpu())
 
 
-@pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 304, 160), (128, 2304, 2048), (200, 1000, 416), (257, 80, 1184), (700, 130, 96)])
+@pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 304, 160), (128, 2304, 2048), (200, 1000, 416), (257, 80, 1184), (700, 130, 96),
+                                   (33, 304, 160), (48, 1000, 416), (64, 2304, 2048)])
 def test_linear_tiled_with_narrow_wave_tiles(M, N, K):
-    """The tiled kernel's wave tiles of 16 and 32 output features (prompts of a few hundred tokens), forced whatever
-    the cost rule would pick: float32 sums whole and in slices of the inner dimension, and the GeGLU epilogue, with
+    """The tiled kernel's wave tiles of 16 and 32 output features (prompts of a few hundred tokens, and 33 to 64
+    tokens where they beat the streaming kernel), forced whatever the cost rule would pick: float32 sums whole and in slices of the inner dimension, and the GeGLU epilogue, with
     token counts that end inside a block, tile counts that a block's four waves do not divide, and inner dimensions
     that are no multiple of a stage."""
     x, w = rnd(M, K, seed=90, dtype=torch.bfloat16), rnd(N, K, seed=91, scale=0.1, dtype=torch.bfloat16)
@@ -807,25 +829,30 @@ def test_projection_with_rotation_and_cache_write_as_its_epilogue(nH, nKV, d, K,
     lens = [int(pos.max()) + 1]
     ang = torch.arange(max(lens), dtype=D)[:, None] * 1e4 ** (-2.0 * torch.arange(d // 2, dtype=D) / d)
     cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    # The separate kernels first; between 33 and 64 tokens with both of the product's kernels, since the fused call
+    # takes the streaming or the tiled one by its rule there (they add up the inner dimension in different orders).
     res = []
-    for fused in (False, True):
-        for frag_in in ((False, True) if fused and K % 32 == 0 else (False,)):
-            kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, n_seq, seed=62)
-            q_out = torch.full((M, nH * d), float("nan"), dtype=torch.bfloat16, device=DEV)
-            if fused:
-                xin = acts_to_fragments(x) if frag_in else x
-                ops.linear_rope_cache(xin, wf, q_out, kp, vp, cos, sin, pos, seq, bt, k_in=K, num_heads=nH, num_kv_heads=nKV,
-                                      head_dim=d, max_position=max(lens) - 1, kv_layout=layout, rows=M,
-                                      x_layout=ops.LAYOUT_FRAG16 if frag_in else ops.LAYOUT_ROW)
-            else:
-                qkv = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-                ops.linear(x, wf, qkv, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, full_precision=False)
-                ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
-                                     rotary_dim=d, max_position=max(lens) - 1, kv_layout=layout, interleaved=True)
-            res.append((q_out, kp, vp))
-    for other in res[1:]:
-        for a, b in zip(res[0], other):
-            assert torch.equal(a, b)
+    cases = [(False, False, ops.LINEAR_AUTO)] + ([(False, False, ops.LINEAR_MFMA)] if 32 < M <= 64 else [])
+    cases += [(True, frag_in, None) for frag_in in ((False, True) if K % 32 == 0 else (False,))]
+    for fused, frag_in, variant in cases:
+        kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, n_seq, seed=62)
+        q_out = torch.full((M, nH * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        if fused:
+            xin = acts_to_fragments(x) if frag_in else x
+            ops.linear_rope_cache(xin, wf, q_out, kp, vp, cos, sin, pos, seq, bt, k_in=K, num_heads=nH, num_kv_heads=nKV,
+                                  head_dim=d, max_position=max(lens) - 1, kv_layout=layout, rows=M,
+                                  x_layout=ops.LAYOUT_FRAG16 if frag_in else ops.LAYOUT_ROW)
+        else:
+            qkv = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            ops.linear(x, wf, qkv, n_out=N, k_in=K, layout=ops.LAYOUT_FRAG16, variant=variant, full_precision=False)
+            ops.rope_cache_write(qkv, q_out, kp, vp, cos, sin, pos, seq, bt, num_heads=nH, num_kv_heads=nKV, head_dim=d,
+                                 rotary_dim=d, max_position=max(lens) - 1, kv_layout=layout, interleaved=True)
+        res.append((fused, (q_out, kp, vp)))
+    separate = [r for f, r in res if not f]
+    for f, other in res:
+        if f:
+            assert any(all(torch.equal(a, b) for a, b in zip(ref, other)) for ref in separate)
+    res = [r for _, r in res]
     # and the separate kernels against the plain formulas, from the rows in their plain order
     qkv_ref = x.double().cpu() @ w.double().cpu().T
     qkv_ref = qkv_ref.to(torch.bfloat16).double()
