@@ -61,11 +61,9 @@ int alice_linear_split_hint_frag(int M, int N, int K) {
   // more than 64 tokens: the tiled kernel's own rule (activations in fragment order, as prompts bring them)
   if (M > 64) return alice_mfma_tiled_plan(M, N, K, ALICE_EPI_NONE, DT_F32, 0, 1).split;
   const int KT = (K + 31) / 32;
-  if (M > 32) {
-    const TiledPlan p = alice_mfma_tiled_plan(M, N, K, ALICE_EPI_NONE, DT_F32, 0, 1);
-    if (p.wn != 0) return p.split;
-    return skinny_split_with_six(M, N, K, KT >= 128 ? 4 : (KT >= 32 ? 2 : 1));
-  }
+  const TiledPlan p = alice_mfma_tiled_plan(M, N, K, ALICE_EPI_NONE, DT_F32, 0, 1);
+  if (p.wn != 0) return p.split;                             // the tiled kernel's narrow tiles are the better ones here
+  if (M > 32) return skinny_split_with_six(M, N, K, KT >= 128 ? 4 : (KT >= 32 ? 2 : 1));
   const int groups = ceil_div(ceil_div(N, 16), alice_mfma_stream_row_tiles_base(M, N, ALICE_EPI_NONE, 1, K));
   int split = 1;
   // aim at about 1024 blocks, keep at least 16 k-tiles (4 per wave) per slice
@@ -89,8 +87,8 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   // blocks for the tiled kernel, which shares the activations through LDS, from 33 tokens on (the 2B head: the same
   // time at 32 tokens, 228 against 277 us at 48; the streaming kernel 198 against 210 us at 17).
   bool skinny = variant == ALICE_LINEAR_SKINNY || (variant == ALICE_LINEAR_AUTO && M <= 64 && !(M > 32 && N >= 65536 && split_k == 1));
-  // 33 to 64 tokens: the tiled kernel's narrow tiles where its rule prefers them
-  if (skinny && variant == ALICE_LINEAR_AUTO && M > 32 && alice_mfma_tiled_plan(M, N, K, epi, y_dtype, split_k, x_layout == ALICE_LAYOUT_FRAG16).wn != 0)
+  // the tiled kernel's narrow tiles where its rule prefers them
+  if (skinny && variant == ALICE_LINEAR_AUTO && alice_mfma_tiled_plan(M, N, K, epi, y_dtype, split_k, x_layout == ALICE_LAYOUT_FRAG16).wn != 0)
     skinny = false;
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
   ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),

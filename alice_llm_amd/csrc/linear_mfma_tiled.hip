@@ -62,13 +62,17 @@ TiledPlan alice_mfma_tiled_plan(int M, int N, int K, int epi, int y_dtype, int s
   const int KT = ceil_div(K, 32), NT = ceil_div(N * (epi == ALICE_EPI_GEGLU ? 2 : 1), 16);
   const bool may_split = epi == ALICE_EPI_NONE && y_dtype == DT_F32;
   if (M <= 64) {
-    // 33 to 64 tokens: the streaming kernel, or the narrow tiles in blocks of 64 tokens with stages of eight
+    // Up to 64 tokens: the streaming kernel, or the narrow tiles in blocks of 64 tokens with stages of eight
     // k-tiles.  Measured on 23 shapes at 33, 40, 48 and 64 tokens: the tiled kernel is 8 to 57 % faster where its
     // blocks come close to one a CU (the most blocks up to 256 over both tiles and the slice counts, the fewest
     // slices among equals), slower where they are few (48 to 80 blocks: 3 to 20 %) or more than 256, and no better
     // with the GeGLU epilogue below 190 blocks; with that rule the mean gain is 13 %, the worst case -3 %.
+    // Up to 32 tokens the streaming kernel is the better one except for float32 sums over a long inner dimension
+    // in slices (output and down projections: 2 to 17 % for the tiled kernel on eight shapes of 16 to 134 MB; a
+    // matrix of 340 MB, which the streaming kernel reads with the streaming hint, is 4 to 10 % slower tiled).
     TiledPlan none{0, 4, 8, split > 0 ? split : 1};
-    if (!(x_frag && M > 32 && narrow_built(epi, y_dtype))) return none;
+    if (!(x_frag && narrow_built(epi, y_dtype))) return none;
+    if (M <= 32 && !(may_split && K >= 4096 && (size_t)N * K < ((size_t)128 << 20))) return none;
     static const int slices[] = {1, 2, 3, 4, 6, 8, 12, 16};
     int best_b = 0, best_wn = 0, best_sp = 0;
     for (int wn = 2; wn >= 1; --wn) {
@@ -79,7 +83,7 @@ TiledPlan alice_mfma_tiled_plan(int M, int N, int K, int epi, int y_dtype, int s
         if (b <= 256 && (b > best_b || (b == best_b && sp < best_sp))) { best_b = b; best_wn = wn; best_sp = sp; }
       }
     }
-    if (best_b >= 190 || (epi != ALICE_EPI_GEGLU && best_b >= 96)) return TiledPlan{best_wn, 4, 8, best_sp};
+    if (best_b >= 190 || (M > 32 && epi != ALICE_EPI_GEGLU && best_b >= 96)) return TiledPlan{best_wn, 4, 8, best_sp};
     return none;
   }
   const int sp0 = split > 0 ? split : (may_split ? tiled_split_wide(M, N, K) : 1);
