@@ -93,10 +93,21 @@ int alice_attention_prefill(const void* q, const void* k_pool, const void* v_poo
                             int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
                             float scale, float softcap, int window, int variant, int out_layout, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
+// out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]
+// = (maximum as a base-2 exponent, sum, two unused, unnormalised output: the output starts at a multiple of 16
+// bytes), for alice_linear_parts to combine.
+#define ALICE_ATTN_PARTS_HEAD 4
 int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                            const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
                            int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
                            int out_layout, hipStream_t stream);
+
+// The output projection straight from the parts of alice_attention_decode (at most 16 sequences, weights in the
+// fragment layout, [N, nH d]): y[slices][M][N] float32 partial sums, slices = alice_linear_parts_split(...), which
+// is 0 where the sizes are not covered.
+int alice_linear_parts_split(int M, int N, int nH, int d, int splits);
+int alice_linear_parts(const float* parts, int splits, int nH, int d, const void* w, float* y, int M, int N,
+                       hipStream_t stream);
 
 // Lowest index among equal maxima.
 int alice_argmax_chunks(int B, int V);

@@ -570,7 +570,7 @@ __global__ __launch_bounds__(64 * NW * KS, NW * KS == 4 ? 2 : 1) void attn_prefi
 // group (group <= 16).  The sequence's 32-key blocks are dealt out in contiguous runs to the
 // splits * 4 waves; every wave keeps a running (max, sum, output); the block's four waves are combined
 // in LDS in the order 0, 1, 2, 3 and the split's result goes to `parts`:
-// [sequence][head][split][D + 2] = (max, sum, unnormalised output).  With one split the output is final.
+// [sequence][head][split][4 + D] = (max, sum, two unused, unnormalised output).  With one split the output is final.
 template <int DT, bool SOFTCAP>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
@@ -659,8 +659,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     if (splits == 1) {
       out[decode_out_index(out_layout, b, head * D + e, nH * D)] = f32_to_bf16(acc / ll);
     } else {
-      float* pr = parts + (((size_t)b * nH + head) * splits + split) * (D + 2);
-      pr[2 + e] = acc;
+      float* pr = parts + (((size_t)b * nH + head) * splits + split) * (D + ALICE_ATTN_PARTS_HEAD);
+      pr[ALICE_ATTN_PARTS_HEAD + e] = acc;
       if (e == 0) { pr[0] = mm; pr[1] = ll; }
     }
   }
@@ -673,11 +673,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits,
                                           int nH, int out_layout) {
   __shared__ float fs[65];
-  const float* pr = parts + (size_t)blockIdx.x * splits * (D + 2);
+  const int PS = D + ALICE_ATTN_PARTS_HEAD;
+  const float* pr = parts + (size_t)blockIdx.x * splits * PS;
   const int t = threadIdx.x;
   if (t < 64) {
-    const float m = t < splits ? pr[(size_t)t * (D + 2)] : -INFINITY;
-    const float l = t < splits ? pr[(size_t)t * (D + 2) + 1] : 0.f;
+    const float m = t < splits ? pr[(size_t)t * PS] : -INFINITY;
+    const float l = t < splits ? pr[(size_t)t * PS + 1] : 0.f;
     const float mm = wave_max(m);
     const float f = (m == -INFINITY) ? 0.f : exp2_fast(m - mm);
     const float ll = wave_sum(l * f);
@@ -691,7 +692,7 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
     for (int s0 = 0; s0 < splits; s0 += 8) {
       float v[8];
 #pragma unroll
-      for (int p = 0; p < 8; ++p) v[p] = (s0 + p < splits) ? pr[(size_t)(s0 + p) * (D + 2) + 2 + e] : 0.f;
+      for (int p = 0; p < 8; ++p) v[p] = (s0 + p < splits) ? pr[(size_t)(s0 + p) * PS + ALICE_ATTN_PARTS_HEAD + e] : 0.f;
 #pragma unroll
       for (int p = 0; p < 8; ++p) acc += v[p] * fs[min(s0 + p, 63)];
     }
@@ -802,7 +803,7 @@ extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const 
 
 // Number of float32 elements `parts` must hold for a decode call.
 extern "C" long alice_attention_decode_workspace(int B, int nH, int d, int splits) {
-  return splits <= 1 ? 0 : (long)B * nH * splits * (d + 2);
+  return splits <= 1 ? 0 : (long)B * nH * splits * (d + ALICE_ATTN_PARTS_HEAD);
 }
 
 extern "C" int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
@@ -814,6 +815,7 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
   ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
   ALICE_CHECK(B >= 0 && nKV <= 65535 && splits >= 1 && splits <= 64, "attention: bad batch B=%d or splits=%d", B, splits);
   ALICE_CHECK(splits == 1 || parts != nullptr, "attention: split keys need the workspace");
+  ALICE_CHECK(out != nullptr || splits > 1, "attention: without an output the keys must be split (the parts are the result)");
   ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
   ALICE_CHECK(out_layout == 0 || out_layout == 1, "attention: unknown output layout %d", out_layout);
   if (B == 0) return 0;
@@ -831,7 +833,7 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
   if (d == 64) GO(2); else if (d == 128) GO(4); else GO(8);
 #undef GO
   ALICE_LAUNCH_CHECK();
-  if (splits > 1) {
+  if (splits > 1 && out != nullptr) {
     attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits, nH, out_layout);
     ALICE_LAUNCH_CHECK();
   }

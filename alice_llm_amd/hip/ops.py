@@ -49,6 +49,8 @@ def _declare(lib) -> None:
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
+        "alice_linear_parts_split": [I, I, I, I, I],
+        "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
         "alice_argmax_chunks": [I, I],
         "alice_sample_workspace": [I, I],
@@ -405,6 +407,7 @@ def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
 
 
 KV_ROW, KV_FRAGMENT = 0, 1
+ATTN_PARTS_HEAD = 4             # floats before a split's output in the parts of attention_decode (ALICE_ATTN_PARTS_HEAD)
 KV_FRAGMENT_PAGE = 64            # positions per page that the fragment layout of keys and values is written for
 ATTENTION_MAX_HEAD_DIM = 256     # the largest head size any attention kernel here takes
 
@@ -461,12 +464,16 @@ def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_ta
 
 def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,
                      scale: float, softcap: Optional[float], window: Optional[int], splits: Optional[int] = None,
-                     out_layout: int = LAYOUT_ROW) -> None:
-    """out_layout FRAG16: `out` is a flat buffer of ceil16(B) * num_heads * d elements in fragment order."""
+                     out_layout: int = LAYOUT_ROW):
+    """out_layout FRAG16: `out` is a flat buffer of ceil16(B) * num_heads * d elements in fragment order.
+    Returns (parts, splits).  With out=None the keys' splits are left uncombined in `parts`
+    ([B, heads, splits, 4 + d] float32, flat) for linear_parts(); that needs splits > 1."""
     n_pages, nKV, page_size, d = k_pool.shape
     B = q.shape[0]
     _dev(q, "q", torch.bfloat16, (B, num_heads * d))
-    if out_layout == LAYOUT_FRAG16:
+    if out is None:
+        pass
+    elif out_layout == LAYOUT_FRAG16:
         _dev(out, "out", torch.bfloat16, (frag_rows(B) * num_heads * d,))
     else:
         _dev(out, "out", torch.bfloat16, (B, num_heads * d))
@@ -479,10 +486,43 @@ def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_h
     if splits is None:
         reach = max_context if not window else min(max_context, window + 32)
         splits = decode_splits(B, nKV, reach)
-    parts = torch.empty((B * num_heads * splits * (d + 2),), dtype=torch.float32, device=q.device) if splits > 1 else None
-    _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
+    if out is None and splits < 2:
+        raise HipLibraryError("attention_decode: without an output buffer the keys must be split")
+    parts = (torch.empty((B * num_heads * splits * (ATTN_PARTS_HEAD + d),), dtype=torch.float32, device=q.device)
+             if splits > 1 else None)
+    _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), None if out is None else out.data_ptr(),
           _opt(parts, "parts"), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], B, num_heads,
           nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, int(out_layout), _stream())
+    return parts, splits
+
+
+def decode_attention_splits(n_seqs: int, num_kv_heads: int, max_context: int, window: Optional[int]) -> int:
+    """The number of key splits that attention_decode picks by itself for a step."""
+    reach = max_context if not window else min(max_context, window + 32)
+    return decode_splits(n_seqs, num_kv_heads, reach)
+
+
+def linear_parts_slices(M: int, n_out: int, num_heads: int, head_dim: int, splits: int) -> int:
+    """Into how many slices linear_parts() cuts the inner dimension for these sizes; 0 where it does not cover them."""
+    return library().alice_linear_parts_split(int(M), int(n_out), int(num_heads), int(head_dim), int(splits))
+
+
+def linear_parts(parts: torch.Tensor, splits: int, w: torch.Tensor, y: torch.Tensor, *, num_heads: int, head_dim: int) -> None:
+    """y[slices, M, n_out] (float32 partial sums) = the output projection of what the uncombined parts of
+    attention_decode combine to, without a kernel for the combine: w is the fragment layout of [n_out, heads * d]."""
+    if y.dim() != 3:
+        raise HipLibraryError("y must be [slices, M, n_out]")
+    slices, M, n_out = y.shape
+    _dev(y, "y", torch.float32)
+    _dev(parts, "parts", torch.float32, (M * num_heads * splits * (ATTN_PARTS_HEAD + head_dim),))
+    _dev(w, "w", torch.bfloat16)
+    need = ((n_out + 15) // 16 * 16) * (num_heads * head_dim)
+    if w.numel() != need:
+        raise HipLibraryError(f"w in fragment layout must hold {need} elements, found {w.numel()}")
+    if slices != linear_parts_slices(M, n_out, num_heads, head_dim, splits) or slices == 0:
+        raise HipLibraryError(f"y must have {linear_parts_slices(M, n_out, num_heads, head_dim, splits)} slices for these sizes (0: not covered)")
+    _call("alice_linear_parts", parts.data_ptr(), int(splits), int(num_heads), int(head_dim), w.data_ptr(), y.data_ptr(),
+          int(M), int(n_out), _stream())
 
 
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,

@@ -101,6 +101,19 @@ class Attention(Part):
                 self.position.rotate_and_store(qkv, q, ctx, cache, pair_order=True, **geometry)
             else:
                 self.position.rotate_and_store(qkv, q, ctx, cache, **geometry)
+        # Single tokens of at most 16 sequences whose keys are split over blocks: the output projection combines the
+        # splits itself (one kernel fewer a layer).
+        if (ctx.is_decode and self.kv_layout == ops.KV_FRAGMENT and self.o.layout == ops.LAYOUT_FRAG16
+                and self.nH // self.nKV <= 16 and getattr(ctx, "fragment_activations", False)):
+            splits = ops.decode_attention_splits(T, self.nKV, ctx.max_context, self.window)
+            slices = ops.linear_parts_slices(T, self.o.n, self.nH, self.d, splits) if splits > 1 else 0
+            if slices > 0:
+                parts, _ = ops.attention_decode(q, cache.k, cache.v, None, ctx.context_lens, cache.block_table,
+                                                num_heads=self.nH, max_context=ctx.max_context, scale=self.scale,
+                                                softcap=self.softcap, window=self.window, splits=splits)
+                y = torch.empty((slices, T, self.o.n), dtype=torch.float32, device=q.device)
+                ops.linear_parts(parts, splits, self.o.weight, y, num_heads=self.nH, head_dim=self.d)
+                return y if slices > 1 else y[0]
         # The matrix-core kernels' output goes to the output projection in fragment order.
         frag = (getattr(ctx, "fragment_activations", False) and self.kv_layout == ops.KV_FRAGMENT
                 and self.o.accepts_fragment_input and FragmentActs.possible(self.precision, T, self.q_dim))
