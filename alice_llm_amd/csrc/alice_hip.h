@@ -102,7 +102,7 @@ int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool
                            int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
                            int out_layout, hipStream_t stream);
 
-// The output projection straight from the parts of alice_attention_decode (at most 16 sequences, weights in the
+// The output projection straight from the parts of alice_attention_decode (at most 16 sequences and 16 splits, weights in the
 // fragment layout, [N, nH d]): y[slices][M][N] float32 partial sums, slices = alice_linear_parts_split(...), which
 // is 0 where the sizes are not covered.
 int alice_linear_parts_split(int M, int N, int nH, int d, int splits);

@@ -43,8 +43,8 @@ __global__ __launch_bounds__(256) void linear_parts_kernel(const float* __restri
 
   // ---- the combined output of the slice: an item is eight consecutive features of one token.  A thread works
   // out the weights of its token's splits itself (the 32 threads of a token and head read the same maxima and sums),
-  // so nothing but the loads stands between the kernel's start and the product; with up to SR splits they are all
-  // in flight at once.
+  // so nothing but the loads stands between the kernel's start and the product; they are all in flight at once
+  // (at most SR splits: with more, which single sequences at long contexts have, the combine stays a kernel).
   const size_t pstride = (size_t)(D + ALICE_ATTN_PARTS_HEAD);
   const int chunks = per * 4;
   for (int it = threadIdx.x; it < 16 * chunks; it += 256) {
@@ -55,62 +55,28 @@ __global__ __launch_bounds__(256) void linear_parts_kernel(const float* __restri
       const float* pr = parts + ((size_t)m * nH + k / D) * S * pstride;
       float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       float ll = 0.f;
-      if (S <= SR) {
-        float2 ml[SR];
-        float4 v[SR][2];
+      float2 ml[SR];
+      float4 v[SR][2];
 #pragma unroll
-        for (int q = 0; q < SR; ++q) {
-          const float* src = pr + (size_t)min(q, S - 1) * pstride;
-          ml[q] = *reinterpret_cast<const float2*>(src);
+      for (int q = 0; q < SR; ++q) {
+        const float* src = pr + (size_t)min(q, S - 1) * pstride;
+        ml[q] = *reinterpret_cast<const float2*>(src);
 #pragma unroll
-          for (int j = 0; j < 2; ++j) v[q][j] = *reinterpret_cast<const float4*>(src + ALICE_ATTN_PARTS_HEAD + e0 + 4 * j);
-        }
-        float mm = -INFINITY;
+        for (int j = 0; j < 2; ++j) v[q][j] = *reinterpret_cast<const float4*>(src + ALICE_ATTN_PARTS_HEAD + e0 + 4 * j);
+      }
+      float mm = -INFINITY;
 #pragma unroll
-        for (int q = 0; q < SR; ++q) mm = fmaxf(mm, ml[q].x);
+      for (int q = 0; q < SR; ++q) mm = fmaxf(mm, ml[q].x);
 #pragma unroll
-        for (int q = 0; q < SR; ++q) {
-          const float f = (q < S && ml[q].x != -INFINITY) ? exp2_hw(ml[q].x - mm) : 0.f;
-          ll += ml[q].y * f;
+      for (int q = 0; q < SR; ++q) {
+        const float f = (q < S && ml[q].x != -INFINITY) ? exp2_hw(ml[q].x - mm) : 0.f;
+        ll += ml[q].y * f;
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            acc[4 * j] += v[q][j].x * f;
-            acc[4 * j + 1] += v[q][j].y * f;
-            acc[4 * j + 2] += v[q][j].z * f;
-            acc[4 * j + 3] += v[q][j].w * f;
-          }
-        }
-      } else {
-        float mm = -INFINITY;
-        for (int s0 = 0; s0 < S; s0 += 8) {
-          float t[8];
-#pragma unroll
-          for (int q = 0; q < 8; ++q) t[q] = pr[(size_t)min(s0 + q, S - 1) * pstride];
-#pragma unroll
-          for (int q = 0; q < 8; ++q) mm = fmaxf(mm, t[q]);
-        }
-        for (int s0 = 0; s0 < S; s0 += 4) {
-          float2 ml[4];
-          float4 v[4][2];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float* src = pr + (size_t)min(s0 + q, S - 1) * pstride;
-            ml[q] = *reinterpret_cast<const float2*>(src);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) v[q][j] = *reinterpret_cast<const float4*>(src + ALICE_ATTN_PARTS_HEAD + e0 + 4 * j);
-          }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float f = (s0 + q < S && ml[q].x != -INFINITY) ? exp2_hw(ml[q].x - mm) : 0.f;
-            ll += ml[q].y * f;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              acc[4 * j] += v[q][j].x * f;
-              acc[4 * j + 1] += v[q][j].y * f;
-              acc[4 * j + 2] += v[q][j].z * f;
-              acc[4 * j + 3] += v[q][j].w * f;
-            }
-          }
+        for (int j = 0; j < 2; ++j) {
+          acc[4 * j] += v[q][j].x * f;
+          acc[4 * j + 1] += v[q][j].y * f;
+          acc[4 * j + 2] += v[q][j].z * f;
+          acc[4 * j + 3] += v[q][j].w * f;
         }
       }
       const float sc = 1.f / ll;
@@ -155,7 +121,7 @@ struct PartsPlan { int wn, split; };
 PartsPlan parts_plan(int M, int N, int nH, int D, int S) {
   PartsPlan none{0, 0};
   const int K = nH * D;
-  if (M < 1 || M > 16 || S < 2 || S > 64 || D % 32 != 0 || N < 1) return none;
+  if (M < 1 || M > 16 || S < 2 || S > 16 || D % 32 != 0 || N < 1) return none;
   const int KT = K / 32, NT = ceil_div(N, 16);
   int most = 0;
   for (int pass = 0; pass < 2; ++pass) {
