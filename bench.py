@@ -4,7 +4,7 @@
 
 A step is one decode step of a batch of 8 sequences that were prefilled with 2,048-token prompts;
 by default the timed steps run the context from 2,048 out to 4,096.  The printed line also holds the
-prefill of one 2,048-token prompt (and of one 8,192-token prompt), the decode step's memory roofline (at the
+prefill of one 2,048-token prompt (and of prompts of 8,192, 512 and 128 tokens), the decode step's memory roofline (at the
 mean context of the timed steps), and decode throughput at batch 1 and 64 over the same range, each with
 its roofline.
 
@@ -82,7 +82,7 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--ids-through-host", action="store_true",
                     help="read every step's chosen ids on the host before the next step is queued (the loop with an observer)")
-    ap.add_argument("--prefill-tokens", default="2048,8192", help="prompt lengths whose prefill is timed (the first is the headline's)")
+    ap.add_argument("--prefill-tokens", default="2048,8192,512,128", help="prompt lengths whose prefill is timed (the first is the headline's)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
