@@ -124,24 +124,39 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
       for (int j = 0; j < MT; ++j) acc[i][j] = mfma16(a[u][i], b[u][j], acc[i][j]);
   }
 
-  if (wave > 0) {
+  // The waves' sums meet in LDS.  A tile of the output (a pair of tiles with GeGLU) has an owner among the waves,
+  // in turn; every other wave leaves its sum of that tile in LDS (its place there: its index among the others), and
+  // the owner adds them up in the order of the waves, its own in its place, and runs the epilogue of its tiles: the
+  // same sums in the same order whoever owns a tile, and the epilogue's arithmetic and stores on all waves at once.
+  constexpr int UNIT = EPI == ALICE_EPI_GEGLU ? 2 : 1;      // row tiles an owner takes together
+  auto owner_of = [&](int i, int j) { return ((i / UNIT) * MT + j) % NW; };
 #pragma unroll
-    for (int i = 0; i < RT; ++i)
+  for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int j = 0; j < MT; ++j)
-        *reinterpret_cast<f32x4*>(red + ((size_t)((wave - 1) * RT * MT + i * MT + j) * 64 + lane) * 4) = acc[i][j];
-  }
-  __syncthreads();
-  if (wave != 0) return;
-#pragma unroll
-  for (int w = 0; w < NW - 1; ++w)
-#pragma unroll
-    for (int i = 0; i < RT; ++i)
-#pragma unroll
-      for (int j = 0; j < MT; ++j) {
-        f32x4 p = *reinterpret_cast<const f32x4*>(red + ((size_t)(w * RT * MT + i * MT + j) * 64 + lane) * 4);
-        acc[i][j] += p;
+    for (int j = 0; j < MT; ++j) {
+      const int own = owner_of(i, j);
+      if (wave != own) {
+        const int slot = wave < own ? wave : wave - 1;
+        *reinterpret_cast<f32x4*>(red + ((size_t)(slot * RT * MT + i * MT + j) * 64 + lane) * 4) = acc[i][j];
       }
+    }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < RT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      if (wave != owner_of(i, j)) continue;
+      const f32x4 mine = acc[i][j];
+      f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const int slot = w < wave ? w : w - 1;
+        const f32x4 p = w == wave ? mine
+                                  : *reinterpret_cast<const f32x4*>(red + ((size_t)(slot * RT * MT + i * MT + j) * 64 + lane) * 4);
+        sum = w == 0 ? p : sum + p;
+      }
+      acc[i][j] = sum;
+    }
 
   if constexpr (EPI == ALICE_EPI_ROPE) {
 #pragma unroll
@@ -150,7 +165,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
       const RopeToken t = rope_token(ra, row[j]);
 #pragma unroll
       for (int i = 0; i < RT; ++i)
-        if (tile[i] < NT) rope_store4(ra, row[j], t, tile[i] * 16 + g * 4, acc[i][j]);
+        if (wave == owner_of(i, j) && tile[i] < NT) rope_store4(ra, row[j], t, tile[i] * 16 + g * 4, acc[i][j]);
     }
     return;
   }
@@ -162,6 +177,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
     if (EPI == ALICE_EPI_GEGLU) {
 #pragma unroll
       for (int p = 0; p < RT / 2; ++p) {
+        if (wave != owner_of(2 * p, j)) continue;
         const int n = (blockIdx.x * (RT / 2) + p) * 16 + g * 4;
         f32x4 o;
 #pragma unroll
@@ -174,6 +190,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
     } else {
 #pragma unroll
       for (int i = 0; i < RT; ++i) {
+        if (wave != owner_of(i, j)) continue;
         const int n = tile[i] * 16 + g * 4;
         f32x4 o;
 #pragma unroll
