@@ -91,7 +91,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   if (skinny && variant == ALICE_LINEAR_AUTO && alice_mfma_tiled_plan(M, N, K, epi, y_dtype, split_k, x_layout == ALICE_LAYOUT_FRAG16).wn != 0)
     skinny = false;
   ALICE_CHECK(!(variant == ALICE_LINEAR_SKINNY && M > 64), "linear: the streaming kernel takes at most 64 rows, found %d", M);
-  ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32 && true),
+  ALICE_CHECK(split_k == 1 || (epi == ALICE_EPI_NONE && y_dtype == DT_F32),
               "linear: partial sums need no epilogue and float32 output");
   ALICE_CHECK(ceil_div(M, 128) <= 65535, "linear: too many rows for one launch (%d)", M);
   ALICE_CHECK(y_layout == ALICE_LAYOUT_ROW || (y_layout == ALICE_LAYOUT_FRAG16 && y_dtype == DT_BF16 && N % 32 == 0 &&
