@@ -13,6 +13,7 @@
 namespace {
 
 constexpr int PARTS_MAX_TILES = 32;   // k-tiles a slice
+constexpr int PARTS_MAX_SLICES = 16;  // slices of the inner dimension: each is a partial result that the add + norm sums
 constexpr int PARTS_U = 8;            // weight k-tiles in flight per wave
 
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -113,8 +114,9 @@ __global__ __launch_bounds__(256) void linear_parts_kernel(const float* __restri
     if (tile[i] < NT) store4(y, row_off, tile[i] * 16 + g * 4, N, acc[i]);
 }
 
-// Slices and tile for M tokens: slices of whole k-tiles, at most PARTS_MAX_TILES of them, whose k-tiles lie in one
-// head each (a head size of a multiple of 32).  Among the choices with at least three quarters of the most blocks
+// Slices and tile for M tokens: at most PARTS_MAX_SLICES slices of whole k-tiles, at most PARTS_MAX_TILES of them,
+// whose k-tiles lie in one head each (a head size of a multiple of 32); inner dimensions that this does not cover
+// (beyond 16,384) are not taken.  Among the choices with at least three quarters of the most blocks
 // that fit the chip once (256), the cheapest by what grows with them: every slice is one more partial result for the
 // add + norm that follows (about 0.12 us), and every block reads its slice's parts anew (about 64 KB a microsecond).
 struct PartsPlan { int wn, split; };
@@ -128,7 +130,7 @@ PartsPlan parts_plan(int M, int N, int nH, int D, int S) {
     PartsPlan best = none;
     float best_cost = 1e30f;
     for (int split = 1; split <= KT; ++split) {
-      if (KT % split != 0 || KT / split > PARTS_MAX_TILES) continue;
+      if (KT % split != 0 || KT / split > PARTS_MAX_TILES || split > PARTS_MAX_SLICES) continue;
       for (int wn = 4; wn >= 1; wn >>= 1) {
         const int b = ceil_div(NT, 4 * wn) * split;
         if (b > 256) continue;

@@ -936,6 +936,33 @@ def test_output_projection_that_combines_the_key_splits_itself(nH, nKV, d, N):
                              window=50, splits=1)
 
 
+def test_many_heads_and_a_narrow_output_keep_the_slices_few():
+    """40 heads of 64 and 24 output features: the rule for the blocks would cut the inner dimension into 80 slices
+    of one k-tile, more partial results than the add + norm that follows sums; it stops at 16."""
+    nH, nKV, d, N, B, splits = 40, 5, 64, 24, 3, 4
+    for n_out in (N, 130, 2304):
+        for M in (1, B, 16):
+            assert 0 <= ops.linear_parts_slices(M, n_out, nH, d, splits) <= 16
+    assert ops.linear_parts_slices(B, N, 128, 256, splits) == 0          # an inner dimension of 32,768: not covered
+    lens = (150, 70, 9)
+    w = rnd(N, nH * d, seed=71, scale=0.1, dtype=torch.bfloat16)
+    wf = ops.to_frag16(w)
+    q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, (1,) * B, None, None, seed=6)
+    slices = ops.linear_parts_slices(B, N, nH, d, splits)
+    assert slices > 0
+    parts, _ = ops.attention_decode(q, kp, vp, None, ctx, bt, num_heads=nH, max_context=max(lens), scale=scale, softcap=None,
+                                    window=None, splits=splits)
+    y = torch.full((slices, B, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.linear_parts(parts, splits, wf, y, num_heads=nH, head_dim=d)
+    close(y.sum(0), ref.double().reshape(B, -1).cpu() @ w.double().cpu().T, 4e-2 * math.sqrt(nH * d / 64), 2 ** -6)
+    # the partial results go through the fused add + norm as the block does it
+    resid = rnd(B, N, seed=72, dtype=torch.float32)
+    w_post = rnd(N, seed=73, dtype=torch.float32)
+    want = resid.double() + P.rms_norm(y.double().sum(0), w_post.double(), 1e-6)
+    ops.add_norm(resid, y, w_post, None, None, eps_post=1e-6, off_post=1.0, n_partials=slices, full_precision=False)
+    close(resid, want, 1e-4, 1e-5)
+
+
 def test_attention_mfma_far_key_and_window_edge():
     nH, nKV, d, L = 4, 2, 64, 700
     def far(b, q, k, v):

@@ -62,6 +62,9 @@ ODD = {
     # query width three times the width, an odd feed-forward width, a scale that is not the head size
     "head-96": dict(_COMMON, num_hidden_layers=1, hidden_size=64, num_attention_heads=2, num_key_value_heads=2, head_dim=96,
                     intermediate_size=17, vocab_size=99, sliding_window=5, query_pre_attn_scalar=7),
+    # forty heads into a width of 24: the output projection's inner dimension is a hundred times its outputs
+    "heads-40": dict(_COMMON, num_hidden_layers=2, hidden_size=24, num_attention_heads=40, num_key_value_heads=5, head_dim=64,
+                     intermediate_size=40, vocab_size=130, sliding_window=50, query_pre_attn_scalar=64),
 }
 
 
