@@ -62,7 +62,6 @@ int alice_linear_split_hint(int M, int N, int K, int w_layout);
 // Rearranges a row-major bfloat16 [N, K] matrix into the fragment layout ([Np/16][Kp/32][64][8],
 // zero padded); dst holds Np * Kp elements with Np = ceil16(N), Kp = ceil32(K).
 int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream);
-int alice_has_mfma_linear();
 int alice_frag16_supported(int rows, int K, int epilogue);
 
 int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool, void* v_pool,

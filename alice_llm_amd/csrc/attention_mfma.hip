@@ -821,17 +821,30 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
   if (B == 0) return 0;
   dim3 grid(B, nKV, splits);
   const size_t lds = (size_t)4 * (nH / nKV) * (d + 4) * sizeof(float);
-#define GO(DT)                                                                                                              \
+  // 16 query heads on a kv head of size 256 take 65 KB for the waves' parts: beyond what a block gets unasked
+  // (the attribute is the kernel's and is told once; a smaller launch is not affected by it)
+#define GO1(DT, CAP)                                                                                                        \
   do {                                                                                                                      \
-    if (softcap > 0.f)                                                                                                      \
-      attn_decode_kernel<DT, true><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits, out_layout);  \
-    else                                                                                                                    \
-      attn_decode_kernel<DT, false><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, \
-          (bf16_t*)out, parts, context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits, out_layout);  \
+    auto kern = attn_decode_kernel<DT, CAP>;                                                                                \
+    if (lds > 48 * 1024) {                                                                                                  \
+      static bool told = false;                                                                                             \
+      if (!told) {                                                                                                          \
+        ALICE_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 4 * 16 * (DT * 32 + 4) * (int)sizeof(float)) == hipSuccess, \
+                    "attention (decode): the device does not give a block %d bytes of LDS", (int)lds);                      \
+        told = true;                                                                                                        \
+      }                                                                                                                     \
+    }                                                                                                                       \
+    kern<<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out, parts,   \
+                                     context_lens, block_table, bt_stride, nH, nKV, scale, softcap, window, splits, out_layout); \
+  } while (0)
+#define GO(DT)                          \
+  do {                                  \
+    if (softcap > 0.f) GO1(DT, true);   \
+    else GO1(DT, false);                \
   } while (0)
   if (d == 64) GO(2); else if (d == 128) GO(4); else GO(8);
 #undef GO
+#undef GO1
   ALICE_LAUNCH_CHECK();
   if (splits > 1 && out != nullptr) {
     attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits, nH, out_layout);

@@ -22,8 +22,6 @@ __global__ void to_frag16_kernel(const bf16_t* __restrict__ src, bf16_t* __restr
 
 }  // namespace
 
-extern "C" int alice_has_mfma_linear() { return 1; }
-
 // Whether a matrix of `rows` x K with this epilogue can use the fragment layout.
 extern "C" int alice_frag16_supported(int rows, int K, int epilogue) {
   if (K % 8 != 0) return 0;                                   // activations are read 8 at a time

@@ -60,6 +60,8 @@ def _declare(lib) -> None:
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = I
+    lib.alice_attention_decode_workspace.argtypes = [I, I, I, I]
+    lib.alice_attention_decode_workspace.restype = L
 
 
 def _open(path: str):
@@ -488,8 +490,8 @@ def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_h
         splits = decode_splits(B, nKV, reach)
     if out is None and splits < 2:
         raise HipLibraryError("attention_decode: without an output buffer the keys must be split")
-    parts = (torch.empty((B * num_heads * splits * (ATTN_PARTS_HEAD + d),), dtype=torch.float32, device=q.device)
-             if splits > 1 else None)
+    parts = (torch.empty((library().alice_attention_decode_workspace(B, num_heads, d, splits),), dtype=torch.float32,
+                         device=q.device) if splits > 1 else None)
     _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), None if out is None else out.data_ptr(),
           _opt(parts, "parts"), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], B, num_heads,
           nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, int(out_layout), _stream())

@@ -715,7 +715,7 @@ def frag_case(nH, nKV, d, lens, new, cap, window, seed, crafted=None):
     return q, kp, vp, bt, i32(cu), i32(list(lens)), torch.cat(refs).reshape(-1, nH * d), scale
 
 
-FRAG_SHAPES = [(6, 2, 64), (4, 4, 64), (8, 4, 256), (4, 1, 128), (3, 3, 128), (32, 16, 128)]
+FRAG_SHAPES = [(6, 2, 64), (4, 4, 64), (8, 4, 256), (4, 1, 128), (3, 3, 128), (32, 16, 128), (16, 1, 256)]
 
 
 def test_fragment_cache_layout_is_what_the_comment_says():
