@@ -40,7 +40,7 @@ def test_embed(wdt):
 
 # ------------------------------------------------------------------ residual add and norms
 @pytest.mark.parametrize("wdt,odt,full", [("float32", "float32", True), ("bfloat16", "bfloat16", False), ("bfloat16", "float32", True)])
-@pytest.mark.parametrize("H", [70, 2304, 5000])
+@pytest.mark.parametrize("H", [70, 400, 2304, 5000, 9000])      # 1, 2, 4 and 8 elements a thread; wider than registers hold
 def test_add_norm_all_forms(wdt, odt, full, H):
     T = 5
     x0 = rnd(T, H, seed=2, scale=3.0)
