@@ -209,8 +209,11 @@ def main() -> int:
                 eng.close(s)
             ms = min(times[1:]) * 1e3
             fl = prefill_flops(cfg, T)
+            # frac: the step's flops over the matrix cores' peak; hbm_frac: the weights, which every step reads once,
+            # over the memory's peak (what bounds a prompt of a few hundred tokens)
             prefills[T] = {"value": round(T / (ms / 1e3), 1), "tokens": T, "ms": round(ms, 3),
-                           "frac": round(fl / (ms / 1e3) / PEAK_FLOPS[short], 4)}
+                           "frac": round(fl / (ms / 1e3) / PEAK_FLOPS[short], 4),
+                           "hbm_frac": round(weight_bytes / (ms / 1e3) / 1e9 / PEAK_HBM_GBS, 4)}
             del eng
             torch.cuda.empty_cache()
             print(f"[bench] prefill {prefills[T]}", file=sys.stderr, flush=True)
