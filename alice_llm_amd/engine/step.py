@@ -275,9 +275,9 @@ class Engine:
         self._graphs = {}
         self._max_graphs = max_graphs
         # short prompt steps are captured too where no part keeps state of its own (a captured step of several
-        # tokens would have to advance such state token by token on the device)
+        # tokens would have to advance such state token by token on the device) and the padding's positions exist
         self._prompt_graphs = {}
-        self.capture_prompts = self.use_graphs and not self.cache.state
+        self.capture_prompts = self.use_graphs and not self.cache.state and self.max_positions >= PROMPT_GRAPH_ROUND
         self._staging = _Staging()
 
     # ------------------------------------------------------------------ sequences
