@@ -277,6 +277,7 @@ class Engine:
         # short prompt steps are captured too where no part keeps state of its own (a captured step of several
         # tokens would have to advance such state token by token on the device) and the padding's positions exist
         self._prompt_graphs = {}
+        self._prompt_seen = {}
         self.capture_prompts = self.use_graphs and not self.cache.state and self.max_positions >= PROMPT_GRAPH_ROUND
         self._staging = _Staging()
 
@@ -347,9 +348,17 @@ class Engine:
             self.cache.commit(slots, n_new)
             return logits
         if self.capture_prompts and want == "last" and B <= PROMPT_GRAPH_SEQS and len(flat) <= PROMPT_GRAPH_TOKENS:
-            logits = self._prompt_graph_step(slots, new_tokens, start)
-            self.cache.commit(slots, n_new)
-            return logits
+            # recorded at a shape's second sighting: shapes that never come back cost nothing
+            key = self._prompt_key(start, n_new)
+            known = key in self._prompt_graphs
+            if not known:
+                self._prompt_seen[key] = self._prompt_seen.pop(key, 0) + 1
+                if len(self._prompt_seen) > 512:
+                    self._prompt_seen.pop(next(iter(self._prompt_seen)))
+            if known or self._prompt_seen[key] >= 2:
+                logits = self._prompt_graph_step(key, slots, new_tokens, start)
+                self.cache.commit(slots, n_new)
+                return logits
 
         cu = [0]
         for n in n_new:
@@ -384,14 +393,17 @@ class Engine:
         return logits
 
     # ------------------------------------------------------------------ captured prompt steps
-    def _prompt_graph_step(self, slots, new_tokens, start) -> torch.Tensor:
+    def _prompt_key(self, start, n_new):
+        """(sequences, tokens rounded up, context bucket, whether the rounding left tokens for the engine's own sequence)"""
+        used = sum(n_new)
+        tokens = -(-used // PROMPT_GRAPH_ROUND) * PROMPT_GRAPH_ROUND
+        reach = max(l + n for l, n in zip(start, n_new))
+        context = min(self.max_positions, -(-reach // CONTEXT_BUCKET) * CONTEXT_BUCKET)
+        return (len(n_new), tokens, context, tokens != used)
+
+    def _prompt_graph_step(self, key, slots, new_tokens, start) -> torch.Tensor:
         """A few short prompts (or pieces) through a captured HIP graph, see _PromptGraph."""
         B = len(slots)
-        used = sum(len(t) for t in new_tokens)
-        tokens = -(-used // PROMPT_GRAPH_ROUND) * PROMPT_GRAPH_ROUND
-        reach = max(l + len(t) for l, t in zip(start, new_tokens))
-        context = min(self.max_positions, -(-reach // CONTEXT_BUCKET) * CONTEXT_BUCKET)
-        key = (B, tokens, context, tokens != used)
         g = self._prompt_graphs.get(key)
         if g is None:
             if len(self._prompt_graphs) >= self._max_graphs:
