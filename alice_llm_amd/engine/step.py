@@ -64,9 +64,11 @@ def _bucket(n: int) -> int:
 
 
 CONTEXT_BUCKET = 512        # captured decode steps are specialised to the context length rounded up to this
-PROMPT_GRAPH_TOKENS = 256   # prompt steps of up to this many tokens are captured as well,
-PROMPT_GRAPH_SEQS = 8       # of at most this many sequences
-PROMPT_GRAPH_ROUND = 16     # their token count rounded up to a multiple of this
+PROMPT_GRAPH_TOKENS = 256   # prompt steps of up to this many tokens are captured as well (beyond, the kernels take
+                            # longer than the host's launches and a replay gains nothing),
+PROMPT_GRAPH_SEQS = 8       # of at most this many sequences,
+PROMPT_GRAPH_ROUND = 16     # their token count rounded up to a multiple of this;
+PROMPT_GRAPH_BUDGET = 2048  # the captured steps kept hold this many tokens together (each keeps its activations)
 
 
 class _Staging:
@@ -78,7 +80,7 @@ class _Staging:
         self.events = [None] * n_buffers
         self.turn = 0
 
-    def upload(self, values: List[int], device) -> torch.Tensor:
+    def upload(self, values: np.ndarray, device) -> torch.Tensor:
         i = self.turn = (self.turn + 1) % len(self.buffers)
         if self.events[i] is not None:
             self.events[i].synchronize()
@@ -86,7 +88,7 @@ class _Staging:
         if self.buffers[i] is None or self.buffers[i].numel() < n:
             self.buffers[i] = torch.empty(max(1024, 2 * n), dtype=torch.int32).pin_memory()
         host = self.buffers[i][:n]
-        host.copy_(torch.tensor(values, dtype=torch.int32))
+        host.numpy()[:] = values
         out = torch.empty(n, dtype=torch.int32, device=device)
         out.copy_(host, non_blocking=True)
         ev = torch.cuda.Event()
@@ -170,7 +172,7 @@ class _PromptGraph:
     """One captured step of a few prompts (or pieces of prompts): B sequences with T tokens in all, unequal.
 
     A short prompt's step is a few hundred launches of kernels that take microseconds; replayed from a graph it takes
-    a third less time at 8 to 32 tokens and 5 % less at 128 to 256 (2B shape).  The graph is recorded for the token
+    a third less time at 8 to 32 tokens and 4 % less at 128 (2B shape).  The graph is recorded for the token
     count rounded up to a multiple of 16 (the matrix products work in tiles of 16 tokens: the padding adds none);
     the tokens beyond the real ones, if any (`spare`), belong to one more sequence, of the engine's own, that lives
     on the cache's spare page, so that no kernel meets a sequence without tokens; what it computes is never read.
@@ -209,13 +211,12 @@ class _PromptGraph:
         B, T = self.n_seqs, self.tokens
         o, sh = self.offs, self.shadow
         n_new = [len(t) for t in new_tokens]
-        flat = [t for seq in new_tokens for t in seq]
-        used = len(flat)
+        used = sum(n_new)
         pad = T - used                                       # the engine's own sequence (none: pad == 0)
         assert (pad > 0) == self.spare and pad >= 0
-        sh[o[0]:o[0] + used] = flat
-        sh[o[1]:o[1] + used] = [l + i for l, n in zip(start, n_new) for i in range(n)]
-        sh[o[2]:o[2] + used] = [b for b, n in enumerate(n_new) for _ in range(n)]
+        sh[o[0]:o[0] + used] = np.concatenate([np.asarray(seq, dtype=np.int64).reshape(-1) for seq in new_tokens])
+        sh[o[1]:o[1] + used] = np.concatenate([np.arange(l, l + n) for l, n in zip(start, n_new)])
+        sh[o[2]:o[2] + used] = np.repeat(np.arange(B), n_new)
         sh[o[3]:o[3] + B] = slots
         cu = np.concatenate(([0], np.cumsum(n_new)))
         sh[o[4]:o[4] + B] = cu[1:] - 1                       # the last token of each sequence
@@ -325,22 +326,19 @@ class Engine:
             if l + n > self.max_positions:
                 raise CacheError(f"slot {s} would reach {l + n} tokens, beyond max_position_embeddings "
                                  f"{self.max_positions}")
-        flat = [int(t) for seq in new_tokens for t in seq]
-        bad = [t for t in flat if not 0 <= t < self.vocab_size]
-        if bad:
-            raise ValueError(f"token id {bad[0]} is outside the vocabulary of {self.vocab_size}")
-        if want == "last":
-            want_lists = [[n - 1] for n in n_new]
-        elif want == "all":
-            want_lists = [list(range(n)) for n in n_new]
-        elif want == "none":
-            want_lists = [[] for _ in n_new]
-        else:
+        # the ids as one array (a prompt of thousands of tokens as Python lists costs the step a millisecond)
+        flat = np.concatenate([np.asarray(seq, dtype=np.int64).reshape(-1) for seq in new_tokens])
+        bad = flat[(flat < 0) | (flat >= self.vocab_size)]
+        if bad.size:
+            raise ValueError(f"token id {int(bad[0])} is outside the vocabulary of {self.vocab_size}")
+        if not isinstance(want, str):
             want_lists = [list(w) for w in want]
             if len(want_lists) != B or any(not 0 <= i < n for w, n in zip(want_lists, n_new) for i in w):
                 raise ValueError("want must give, per sequence, indices into its new tokens")
             if want_lists == [[n - 1] for n in n_new]:
                 want = "last"                                  # said with indices: the same step
+        elif want not in ("last", "all", "none"):
+            raise ValueError('want is "last", "all", "none" or, per sequence, indices into its new tokens')
         self.cache.reserve(slots, n_new)                       # raises before any launch
 
         if self.use_graphs and want == "last" and max(n_new) == 1:
@@ -364,16 +362,23 @@ class Engine:
         for n in n_new:
             cu.append(cu[-1] + n)
         T = cu[-1]
-        positions = [l + i for l, n in zip(start, n_new) for i in range(n)]
-        seq_of = [b for b, n in enumerate(n_new) for _ in range(n)]
-        rows = [cu[b] + i for b, w in enumerate(want_lists) for i in w]
+        positions = np.concatenate([np.arange(l, l + n) for l, n in zip(start, n_new)])
+        seq_of = np.repeat(np.arange(B), n_new)
+        if want == "last":
+            rows = [c - 1 for c in cu[1:]]
+        elif want == "all":
+            rows = np.arange(T)
+        elif want == "none":
+            rows = []
+        else:
+            rows = [cu[b] + i for b, w in enumerate(want_lists) for i in w]
         ctx_lens = [l + n for l, n in zip(start, n_new)]
         width = self.cache.table_width(slots)
         tables = [self.cache.block_table_rows(g, slots, width) for g in range(len(self.cache.groups))]
 
         # one host-to-device copy for all the small integer arrays of the step
         pieces = [flat, positions, seq_of, list(slots), rows, cu, ctx_lens] + [sum(t, []) for t in tables]
-        packed = self._staging.upload(sum(pieces, []), self.device)
+        packed = self._staging.upload(np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in pieces]), self.device)
         offs = [0]
         for p in pieces:
             offs.append(offs[-1] + len(p))
@@ -382,12 +387,12 @@ class Engine:
         if device_tokens is not None:
             part(0).copy_(device_tokens)
         ctx = StepContext(tokens=part(0), positions=part(1), seq_of_token=part(2), slots=part(3),
-                          want_rows=part(4) if rows else None, cu_seqlens=part(5), context_lens=part(6),
+                          want_rows=part(4) if len(rows) else None, cu_seqlens=part(5), context_lens=part(6),
                           n_tokens=T, n_seqs=B, is_decode=all(n == 1 for n in n_new), max_new=max(n_new),
                           max_context=max(ctx_lens), max_position=max(ctx_lens) - 1,
                           new_lens=n_new, start_lens=start, slot_ids=list(slots),
                           fragment_activations=self.model.precision.act == torch.bfloat16,
-                          want_every_row=rows == list(range(T)))
+                          want_every_row=len(rows) == T and (want == "all" or list(rows) == list(range(T))))
         logits = self.model.forward(ctx, self.cache, block_tables)
         self.cache.commit(slots, n_new)
         return logits
@@ -406,7 +411,8 @@ class Engine:
         B = len(slots)
         g = self._prompt_graphs.get(key)
         if g is None:
-            if len(self._prompt_graphs) >= self._max_graphs:
+            while self._prompt_graphs and (len(self._prompt_graphs) >= self._max_graphs or
+                                           sum(k[1] for k in self._prompt_graphs) + key[1] > PROMPT_GRAPH_BUDGET):
                 self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
             g = self._prompt_graphs[key] = _PromptGraph(self, *key)
         else:

@@ -4,6 +4,7 @@ import pytest
 import torch
 
 import alice_llm_amd as alice
+import alice_llm_amd.engine.step as step_mod
 from helpers import TINY, TOL, max_err, model_folder, plain_model, random_tokens
 
 pytestmark = pytest.mark.gpu
@@ -205,7 +206,7 @@ def test_captured_decode_steps_match_eager_on_every_replay(name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", [("tiny-c", "bfloat16"), ("tiny-b", "float32"), ("tiny-a", "bfloat16")])
-def test_captured_prompt_steps_match_eager_and_plain_on_every_replay(name, dtype):
+def test_captured_prompt_steps_match_eager_and_plain_on_every_replay(name, dtype, monkeypatch):
     """Steps of a few short prompts, or pieces of prompts, are recorded into HIP graphs as well (their token count
     rounded up, the tokens beyond the real ones on a sequence of the engine's own), from a shape's second sighting on.
     One graph serves every split of its tokens over its sequences: the same shape comes back with other splits, other
@@ -259,7 +260,7 @@ def test_captured_prompt_steps_match_eager_and_plain_on_every_replay(name, dtype
     keys = set(graph._prompt_graphs)
     assert len(keys) < len(rounds) + 3 and all(g.graph is not None for g in graph._prompt_graphs.values())
     assert {(2, 16, 512, True), (8, 32, 512, True), (2, 64, 512, True), (2, 192, 512, True), (1, 64, 512, True)} <= keys
-    # longer prompts, other wanted rows and shapes seen once are not recorded
+    # other wanted rows and shapes seen once are not recorded
     n = len(keys)
     for again in range(3):                                   # a multiple of 16 tokens: no sequence of the engine's own
         toks = random_tokens(plain.V, 256 + 3, 3 + again)
@@ -273,14 +274,26 @@ def test_captured_prompt_steps_match_eager_and_plain_on_every_replay(name, dtype
     for again in range(3):
         graph.step(s, [random_tokens(plain.V, 9, 4)], "all")
     graph.close(s)
-    for again in range(3):
-        s = graph.open(1)
-        graph.step(s, [random_tokens(plain.V, 257, 3)], "last")
-        graph.close(s)
     s = graph.open(1)
     graph.step(s, [random_tokens(plain.V, 100, 3)], "last")      # seen once
     graph.close(s)
     assert len(graph._prompt_graphs) == n + 2
+    # the recorded steps kept hold a budget of tokens together (each keeps its activations): the oldest go
+    monkeypatch.setattr(step_mod, "PROMPT_GRAPH_BUDGET", 300)
+    for again in range(3):
+        toks = random_tokens(plain.V, 200, 8 + again)
+        ref = plain.forward(toks)
+        s = graph.open(1)
+        assert max_err(graph.step(s, [toks], "last")[0], ref[199]) < tol(dtype, ref)
+        graph.close(s)
+    assert (1, 208, 512, True) in graph._prompt_graphs and sum(k[1] for k in graph._prompt_graphs) <= 300
+    assert len(graph._prompt_graphs) < n
+    # beyond 256 tokens a step's kernels take longer than the host's launches: not recorded
+    for again in range(3):
+        s = graph.open(1)
+        graph.step(s, [random_tokens(plain.V, 257, 3)], "last")
+        graph.close(s)
+    assert all(k[1] <= 256 for k in graph._prompt_graphs)
 
 
 @pytest.mark.parametrize("name,dtype", [("tiny-c", "bfloat16"), ("tiny-b", "float32")])
