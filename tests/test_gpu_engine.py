@@ -156,6 +156,13 @@ def test_step_argument_errors():
         eng.step(s, [[1], [256]])
     with pytest.raises(ValueError, match="at least one token"):
         eng.step(s, [[1], []])
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.step(s, [[1, 2, -1], [3]])
+    with pytest.raises(ValueError, match="want"):
+        eng.step(s, [[1], [2]], "first")
+    with pytest.raises(ValueError, match="want"):
+        eng.step(s, [[1], [2]], [[0], [1]])
+    assert eng.length(s[0]) == 0 and eng.length(s[1]) == 0        # nothing of a refused step stays
     with pytest.raises(alice.CacheError, match="full"):
         eng.step(s, [[1] * 70, [2] * 70])
     with pytest.raises(alice.CacheError, match="max_position"):
