@@ -66,7 +66,7 @@ def _bucket(n: int) -> int:
 CONTEXT_BUCKET = 512        # captured decode steps are specialised to the context length rounded up to this
 PROMPT_GRAPH_TOKENS = 256   # prompt steps of up to this many tokens are captured as well (beyond, the kernels take
                             # longer than the host's launches and a replay gains nothing),
-PROMPT_GRAPH_SEQS = 8       # of at most this many sequences,
+PROMPT_GRAPH_SEQS = 16      # of at most this many sequences,
 PROMPT_GRAPH_ROUND = 16     # their token count rounded up to a multiple of this;
 PROMPT_GRAPH_BUDGET = 2048  # the captured steps kept hold this many tokens together (each keeps its activations)
 
