@@ -10,5 +10,5 @@ from .weights.safetensors_io import WeightFileError
 from .cache import Cache, CacheError
 from .api import Model, load, sample, GenerationResult
 from .engine.step import Engine
-from .engine.generate import Generator
+from .engine.generate import Generator, plan_prompt_steps, run_prompt_steps
 from .sampling import Sampler

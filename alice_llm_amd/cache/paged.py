@@ -79,6 +79,8 @@ class PageGroup:
         if need.page_size is not None and need.page_size != page_size:
             raise CacheError(f"the layers {self.layers} need pages of {need.page_size} positions (their kernels are "
                              f"written for that), the cache has pages of {page_size}")
+        dtype = need.dtype or dtype                 # the mixer's own choice, else the run's activation dtype
+        self.dtype = dtype
         shape = (len(self.layers), n_pages + 1, need.num_kv_heads, page_size)
         self.k = torch.zeros(shape + (need.head_dim,), dtype=dtype, device=device) if allocate else None
         self.v = torch.zeros(shape + (need.v_dim,), dtype=dtype, device=device) if allocate else None

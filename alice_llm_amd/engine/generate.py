@@ -1,7 +1,9 @@
 """The generation loop above the step function: batches of unequal prompts, stop tokens, sequences
 that end earlier, and as many batches one after another as there are requests.
 
-A batch starts together: one step runs all its prompts, then every live sequence gets one token per
+A batch starts together: its prompts run in one ragged step, or, when they hold more tokens than a step's
+budget, in several (a long prompt in pieces, logits asked for at its last piece only; the reference runs its
+prompts request by request, llama3.rs:17783-17795); then every live sequence gets one token per
 step.  A sequence ends when it draws a stop token (which is not part of its output, as in the
 reference, llama3.rs:16137-16139) or reaches its own cap of new tokens (llama3.rs:17813-17835); it
 leaves the batch at once and its slot goes back to the cache, where the next batch takes it.
@@ -66,6 +68,53 @@ def plan_batches(prompt_lens: Sequence[int], caps: Sequence[int], *, max_batch: 
     return batches
 
 
+MAX_STEP_TOKENS = 16384     # a prompt step's activations grow with its tokens (the gated product of the widest
+                            # shape here takes 147 KB a token): 16,384 tokens keep them near 2 GB, and the
+                            # matrix products are as fast per token from 8,192 tokens on
+
+
+def plan_prompt_steps(prompt_lens: Sequence[int], max_step_tokens: Optional[int]) -> List[List[tuple]]:
+    """Cut the prompts of a batch, in order, into steps of at most max_step_tokens tokens (None: one step).
+    A step is a list of (index of the sequence in the batch, first token, number of tokens); a prompt that does
+    not fit into what is left of a step goes on in the next one, so every step but the last is full.  A sequence
+    appears at most once in a step, and its pieces come in consecutive steps."""
+    if max_step_tokens is not None and max_step_tokens < 1:
+        raise ValueError("a prompt step needs room for at least one token")
+    budget = max_step_tokens or sum(prompt_lens) or 1
+    steps: List[List[tuple]] = []
+    cur: List[tuple] = []
+    room = budget
+    for i, n in enumerate(prompt_lens):
+        at = 0
+        while at < n:
+            take = min(n - at, room)
+            cur.append((i, at, take))
+            at += take
+            room -= take
+            if room == 0:
+                steps.append(cur)
+                cur, room = [], budget
+    if cur:
+        steps.append(cur)
+    return steps
+
+
+def run_prompt_steps(engine, slots: Sequence[int], prompts: Sequence[Sequence[int]],
+                     max_step_tokens: Optional[int] = MAX_STEP_TOKENS):
+    """Run the prompts of sequences that start together, in as many ragged steps as the budget asks for; returns
+    the logits at every prompt's last token, in the order of the sequences."""
+    steps = plan_prompt_steps([len(p) for p in prompts], max_step_tokens)
+    if len(steps) == 1:
+        return engine.step(list(slots), [list(p) for p in prompts], "last")
+    rows = []
+    for step in steps:
+        want = [[n - 1] if at + n == len(prompts[i]) else [] for i, at, n in step]
+        logits = engine.step([slots[i] for i, _, _ in step], [list(prompts[i][at:at + n]) for i, at, n in step], want)
+        if any(want):
+            rows.append(logits)
+    return rows[0] if len(rows) == 1 else torch.cat(rows)
+
+
 class Generator:
     """Runs requests through an engine.  `engine` needs open(n), step(slots, tokens, want) and
     close(slots) and a cache with `max_tokens` and `slots.n_slots`; `sampler(logits, requests, draws)`
@@ -74,8 +123,9 @@ class Generator:
     def __init__(self, engine, *, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
                  stop_token_ids: Sequence[int] = (), max_batch: Optional[int] = None,
                  sampler: Optional[Callable] = None, include_stop_token: bool = False,
-                 observer: Optional[Callable] = None):
-        """observer(requests, positions, logits, tokens), if given, is called after every step of every batch
+                 observer: Optional[Callable] = None, max_step_tokens: Optional[int] = MAX_STEP_TOKENS):
+        """max_step_tokens: the most tokens of prompts that one step runs (None: a batch's prompts in one step).
+        observer(requests, positions, logits, tokens), if given, is called after every step of every batch
         with the live requests' indices, the position each row's logits belong to, the step's float32 logits
         [rows, vocab] and the token ids drawn from them: what a logits dump of the real run needs."""
         self.engine = engine
@@ -87,6 +137,8 @@ class Generator:
         self.max_batch = max_batch
         self.include_stop_token = include_stop_token
         self.observer = observer
+        self.max_step_tokens = max_step_tokens
+        plan_prompt_steps([], max_step_tokens)                   # refuses a budget below one token
 
     def run(self, prompts: Sequence[Sequence[int]], max_new_tokens: Sequence[int]) -> List[GenerationResult]:
         if len(prompts) != len(max_new_tokens):
@@ -127,7 +179,7 @@ class Generator:
             rows = list(live)                                # the requests of the step whose ids are on their way
             drawn = None                                     # that step's ids on the device and, later, on the host
             if rows:
-                logits = eng.step([slots[r] for r in rows], [list(prompts[r]) for r in rows], "last")
+                logits = run_prompt_steps(eng, [slots[r] for r in rows], [prompts[r] for r in rows], self.max_step_tokens)
                 drawn = self._draw(logits, rows, out, 0)
             first = True
             while rows:

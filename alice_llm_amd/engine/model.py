@@ -51,10 +51,10 @@ class CausalLM:
                                      f"an earlier entry with a cache of its own")
                 a, b = self._need(e.layer), self._need(plan.schedule[e.cache_from].layer)
                 if a is None or b is None or a.kv is None or b.kv is None or \
-                        (a.kv.num_kv_heads, a.kv.head_dim, a.kv.v_dim) != (b.kv.num_kv_heads, b.kv.head_dim, b.kv.v_dim) or \
+                        (a.kv.num_kv_heads, a.kv.head_dim, a.kv.v_dim, a.kv.dtype) != (b.kv.num_kv_heads, b.kv.head_dim, b.kv.v_dim, b.kv.dtype) or \
                         (b.kv.window is not None and (a.kv.window is None or a.kv.window > b.kv.window)):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.cache_from}: "
-                                     f"its keys differ in shape or reach further back than that cache keeps")
+                                     f"its keys differ in shape or dtype, or reach further back than that cache keeps")
         self._loaded = False
 
     # ------------------------------------------------------------------ parameters
@@ -110,6 +110,16 @@ class CausalLM:
             parts += [layer.mixer, layer.feed_forward, layer.block] + list(layer.norms.values())
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
+    def prompt_graph_safe(self) -> bool:
+        """Whether steps of several tokens a sequence can be recorded too: every part that keeps state of its own
+        (a cache need with state tensors) declares `graph_safe_prompts = True`, that is, it advances its state
+        token by token on the device, from ctx.cu_seqlens and ctx.seq_of_token, never from the host copies."""
+        for e in self.plan.schedule:
+            need = self._need(e.layer)
+            if need is not None and need.state and not getattr(self.layers[e.layer].mixer, "graph_safe_prompts", False):
+                return False
+        return True
+
     # ------------------------------------------------------------------ cache needs
     def _need(self, layer: int):
         mixer = self.layers[layer].mixer
@@ -124,7 +134,7 @@ class CausalLM:
         """Runs the step's tokens through the schedule; returns float32 logits at ctx.want_rows."""
         if not self._loaded:
             raise RuntimeError("the model has no weights yet")
-        stream = ResidualStream(self.embedding.forward(ctx.tokens), self.precision)
+        stream = ResidualStream(self.embedding.forward(ctx), self.precision)
         for i, entry in enumerate(self.plan.schedule):
             view = cache.view(i, block_tables, read_from=entry.cache_from)
             self.layers[entry.layer].block.forward(stream, ctx, view)

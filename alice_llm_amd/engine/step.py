@@ -264,6 +264,7 @@ class Engine:
             max_tokens = sum(-(-int(n) // page_size) * page_size for n in seq_lens)
             if max_seqs is None:
                 max_seqs = len(seq_lens)
+        # (the activation dtype is the pages' dtype unless a mixer's KVNeed names another)
         self.cache = Cache(model.cache_needs(), max_tokens=max_tokens, dtype=model.precision.act,
                            device=self.device, max_seqs=max_seqs, page_size=page_size)
         self.vocab_size = model.plan.vocab_size
@@ -275,11 +276,12 @@ class Engine:
         self.use_graphs = safe if use_graphs is None else (use_graphs and safe)
         self._graphs = {}
         self._max_graphs = max_graphs
-        # short prompt steps are captured too where no part keeps state of its own (a captured step of several
-        # tokens would have to advance such state token by token on the device) and the padding's positions exist
+        # short prompt steps are captured too where the padding's positions exist and every part that keeps state
+        # of its own says that it advances that state on the device in steps of several tokens
         self._prompt_graphs = {}
         self._prompt_seen = {}
-        self.capture_prompts = self.use_graphs and not self.cache.state and self.max_positions >= PROMPT_GRAPH_ROUND
+        self.capture_prompts = (self.use_graphs and model.prompt_graph_safe()
+                                and self.max_positions >= PROMPT_GRAPH_ROUND)
         self._staging = _Staging()
 
     # ------------------------------------------------------------------ sequences

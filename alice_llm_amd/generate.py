@@ -5,7 +5,8 @@ Option names and meanings follow the reference's generate examples where it has 
 examples/generate_gpu.rs:31-40; temperature 0 is greedy, generate_gpu.rs:122; --logits-dump N writes,
 for every request, the top-5 logits of its first N generated positions as JSON lines to stderr while the
 request runs: the logits of the run's own steps and the token its sampler drew from them,
-examples/elyza_gguf.rs:31-76, 200-259).  There is no tokenizer here: prompts are token ids, and so is the
+examples/elyza_gguf.rs:31-76, 200-259; --dump-logits FILE sends the same lines to a file instead, for
+every generated position unless --logits-dump N limits them).  There is no tokenizer here: prompts are token ids, and so is the
 output.  The closing lines are the reference's (examples/elyza_gguf.rs:277-286).
 """
 from __future__ import annotations
@@ -40,8 +41,13 @@ def main(argv=None) -> int:
     ap.add_argument("--max-batch", type=int, default=None, help="most sequences in one batch")
     ap.add_argument("--logits-dump", type=int, default=0,
                     help="dump the top-5 logits of each request's first N generated positions (JSON lines on stderr)")
+    ap.add_argument("--dump-logits", metavar="FILE", default=None,
+                    help="write the dump's JSON lines to FILE instead of stderr (every generated position, or the "
+                         "first N with --logits-dump N)")
     ap.add_argument("--ignore-unexpected-tensors", action="store_true",
                     help="tensors in the folder that the model does not declare are warned about instead of refused")
+    ap.add_argument("--keep-stored-dtype", action="store_true",
+                    help="with --dtype bfloat16: matrices stored in float32 stay float32 instead of being rounded once at load")
     args = ap.parse_args(argv)
 
     import alice_llm_amd as alice
@@ -61,18 +67,28 @@ def main(argv=None) -> int:
         else:
             ap.error("--random-weights needs --preset or --config")
         print(f"Building random weights (seed {args.weights_seed})", flush=True)
-        model = alice.load(raw, dtype=args.dtype, random_seed=args.weights_seed)
+        model = alice.load(raw, dtype=args.dtype, random_seed=args.weights_seed, keep_stored_dtype=args.keep_stored_dtype)
     else:
         if not args.model:
             ap.error("give --model DIR, or --random-weights with --preset/--config")
         print(f"Loading model: {args.model}", flush=True)
-        model = alice.load(args.model, dtype=args.dtype, strict=not args.ignore_unexpected_tensors)
+        model = alice.load(args.model, dtype=args.dtype, strict=not args.ignore_unexpected_tensors,
+                           keep_stored_dtype=args.keep_stored_dtype)
 
     stop = _ids(args.stop_ids) if args.stop_ids is not None else None
-    results = model.generate(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
-                             top_k=args.top_k, top_p=args.top_p, seed=args.seed, stop_token_ids=stop,
-                             max_batch=args.max_batch,
-                             observer=_logits_dumper(args.logits_dump) if args.logits_dump > 0 else None)
+    observer = dump_file = None
+    if args.dump_logits:
+        dump_file = open(args.dump_logits, "w")
+        observer = _logits_dumper(args.logits_dump if args.logits_dump > 0 else None, dump_file)
+    elif args.logits_dump > 0:
+        observer = _logits_dumper(args.logits_dump, sys.stderr)
+    try:
+        results = model.generate(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
+                                 top_k=args.top_k, top_p=args.top_p, seed=args.seed, stop_token_ids=stop,
+                                 max_batch=args.max_batch, observer=observer)
+    finally:
+        if dump_file is not None:
+            dump_file.close()
     for i, r in enumerate(results):
         print(f"[{i}] " + ",".join(str(t) for t in r.tokens) + f"  ({r.finish_reason})")
     print("---")
@@ -91,14 +107,15 @@ def main(argv=None) -> int:
     return 0
 
 
-def _logits_dumper(n: int):
-    """An observer of the generation loop: for each request's first n generated positions one JSON line with
-    the request, the position the logits belong to, the token drawn there and the five largest logits."""
+def _logits_dumper(n, out):
+    """An observer of the generation loop: for each request's first n generated positions (n None: all of them)
+    one JSON line to `out` with the request, the position the logits belong to, the token drawn there and the
+    five largest logits."""
     import torch
     seen = {}
 
     def observe(requests, positions, logits, tokens) -> None:
-        rows = [i for i, r in enumerate(requests) if seen.get(r, 0) < n]
+        rows = [i for i, r in enumerate(requests) if n is None or seen.get(r, 0) < n]
         if not rows:
             return
         top = torch.topk(logits[rows], min(5, logits.shape[1]), dim=-1)
@@ -108,7 +125,7 @@ def _logits_dumper(n: int):
             seen[r] = seen.get(r, 0) + 1
             print(json.dumps({"request": r, "position": positions[i], "token": int(tokens[i]),
                               "top5": [[int(t), float(v)] for t, v in zip(indices[j], values[j])]}),
-                  file=sys.stderr, flush=True)
+                  file=out, flush=True)
     return observe
 
 

@@ -69,9 +69,9 @@ class Attention(Part):
             raise KeyError(name)
 
     def finalize(self) -> None:
-        q, k, v = (self._parts.pop(n + "_proj.weight") for n in "qkv")
+        q, k, v = (self.precision.matrix(self._parts.pop(n + "_proj.weight")) for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = q.float(), k.float(), v.float()       # one stored in 32-bit: the fused matrix stays 32-bit
+            q, k, v = q.float(), k.float(), v.float()       # kept as stored, one of them in 32-bit: the fused matrix is 32-bit
         w = torch.cat([q, k, v], dim=0)                     # rows: all q heads, then k heads, then v heads
         # a position encoding may ask for the rows of the q and k heads in another order (rotated pairs next to
         # each other), so that its rotation can be the projection's epilogue

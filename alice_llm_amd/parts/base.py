@@ -21,22 +21,35 @@ class Precision:
     bfloat16: matrix operands, activations between kernels and the cache are bfloat16; sums,
     softmax, norms, rotation and the residual stream are 32-bit.
     float32: everything is 32-bit, with full-precision tanh/exp/sqrt and no matrix-core shortcut.
+
+    keep_stored: on the bfloat16 path a matrix that its file stores in 32-bit is rounded to bfloat16 once, at
+    load, so that it runs on the matrix cores like any other (the reference converts its stored formats once at
+    load too, llama3.rs:12889-12890, 18226-18240); with keep_stored it stays 32-bit and its products run on the
+    plain kernel.  Norm weights always stay as stored.
     """
     name: str
     act: torch.dtype
     full: bool
+    keep_stored: bool = False
 
     @staticmethod
-    def of(name) -> "Precision":
+    def of(name, keep_stored: bool = False) -> "Precision":
         if isinstance(name, Precision):
             return name
         key = {"bf16": "bfloat16", "fp32": "float32", torch.bfloat16: "bfloat16",
                torch.float32: "float32"}.get(name, name)
         if key == "bfloat16":
-            return Precision("bfloat16", torch.bfloat16, False)
+            return Precision("bfloat16", torch.bfloat16, False, bool(keep_stored))
         if key == "float32":
-            return Precision("float32", torch.float32, True)
+            return Precision("float32", torch.float32, True, bool(keep_stored))
         raise ValueError(f"unknown dtype '{name}': bfloat16 or float32")
+
+    def matrix(self, w: torch.Tensor) -> torch.Tensor:
+        """A matrix weight in the dtype in which this run keeps it: as stored, except that the bfloat16 path
+        rounds a matrix stored in 32-bit to bfloat16 (unless keep_stored)."""
+        if self.name == "bfloat16" and not self.keep_stored and w.dtype == torch.float32:
+            return w.to(torch.bfloat16)
+        return w
 
 
 # --------------------------------------------------------------------------- activations in fragment order
@@ -101,12 +114,15 @@ class KVNeed:
     """Keys and values that grow with the sequence: per position, num_kv_heads rows of head_dim keys and of
     value_head_dim values (None: the same as the keys); `window` keys back from the newest are ever read
     (None: all of them).  `page_size`: the number of positions per page that the mixer's kernels are written
-    for (None: any); a cache built with another page size refuses the mixer when the model is put together."""
+    for (None: any); a cache built with another page size refuses the mixer when the model is put together.
+    `dtype`: the dtype of the pages (None: the run's activation dtype); a mixer that wants its keys in 32-bit
+    under bfloat16 activations says so here, and its layers get storage of their own."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_head_dim: Optional[int] = None
     page_size: Optional[int] = None
+    dtype: Optional[torch.dtype] = None
 
     @property
     def v_dim(self) -> int:

@@ -36,7 +36,11 @@ class Embedding(Part):
     def weight_bytes(self) -> int:
         return self.table.nbytes()
 
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx) -> torch.Tensor:
+        """The float32 rows that start the residual stream, one per token of the step.  An embedding sees the
+        whole step (`ctx`: token ids, positions, the sequence of each token), so that one that adds a learned
+        row per position, say, needs nothing else; this one reads the ids only."""
+        tokens = ctx.tokens
         out = torch.empty((tokens.numel(), self.dim), dtype=torch.float32, device=tokens.device)
         ops.embed(tokens, self.table.weight, out, self.scale, self.V, self.dim, self.table.layout)
         return out

@@ -44,7 +44,7 @@ class GatedMLP(Part):
             raise KeyError(name)
 
     def finalize(self) -> None:
-        g, u = self._parts.pop("gate_proj.weight"), self._parts.pop("up_proj.weight")
+        g, u = (self.precision.matrix(self._parts.pop(n + "_proj.weight")) for n in ("gate", "up"))
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.gate_up.load(torch.cat([g, u], dim=0))

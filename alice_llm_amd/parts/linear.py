@@ -1,9 +1,10 @@
 """A dense projection y = x W^T: the building brick of mixers, feed-forwards and the head.
 
 Orientation as in the reference: W is [out, in] row-major and y[r] = sum_c W[r, c] x[c]
-(gguf.rs:4063-4074).  The bfloat16 path rearranges bfloat16 weights once, at load, into the
-fragment layout that the MFMA kernels read; a weight stored in 32-bit stays row-major 32-bit
-and runs on the plain kernel.
+(gguf.rs:4063-4074).  The bfloat16 path rounds a weight stored in 32-bit to bfloat16 and rearranges
+it once, at load, into the fragment layout that the MFMA kernels read (llama3.rs:12889-12890 converts
+once at load as well); only when the run was asked to keep stored dtypes does such a weight stay
+row-major 32-bit and run on the plain kernel.
 """
 from __future__ import annotations
 
@@ -38,6 +39,7 @@ class Linear:
         """Takes a row-major [rows, in] device tensor in its stored dtype."""
         if tuple(w.shape) != (self.weight_rows, self.k):
             raise ValueError(f"weight must be {(self.weight_rows, self.k)}, found {tuple(w.shape)}")
+        w = self.precision.matrix(w)
         if (USE_FRAGMENT_LAYOUT and self.precision.name == "bfloat16" and w.dtype == torch.bfloat16
                 and ops.fragment_layout_supported(self.weight_rows, self.k, self.epilogue)):
             self.weight = ops.to_frag16(w.contiguous())

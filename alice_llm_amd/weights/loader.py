@@ -2,8 +2,11 @@
 
 Every tensor the model declares is looked up by its full name; its shape and dtype are checked
 against the declaration; all problems of a folder (missing and unexpected tensors, wrong shapes,
-dtypes without a kernel) are gathered into one error.  Floating-point tensors stay as stored:
-bfloat16 stays bfloat16 and float32 stays float32; integer tables become int32.  The reference
+dtypes without a kernel) are gathered into one error.  Tensors reach the parts as stored: bfloat16
+as bfloat16, float32 as float32, integer tables as int32.  What a part then keeps is its own matter: norm
+weights stay as stored on every path; the bfloat16 path rounds a matrix stored in float32 to bfloat16 once,
+when it is put into the layout its kernels read, unless the run keeps stored dtypes (Precision.keep_stored).
+The reference
 derives shapes from its configuration and trusts them (llama3.rs:18226-18240) and reports a
 missing tensor by returning None (llama3.rs:12887-12906); its newer loaders name the tensor
 (llama3.rs:1137-1175), which is the behaviour kept here.

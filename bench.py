@@ -113,7 +113,7 @@ def main() -> int:
         torch.cuda.synchronize()
 
     def decode_run(lens, steps, warmup):
-        """Prefill prompts of these lengths (a few sequences per ragged step), then time `steps` decode steps
+        """Prefill prompts of these lengths (in the generation loop's ragged steps), then time `steps` decode steps
         (greedy, tokens fed back).  Returns the time and every sequence's context at the first and after the
         last timed step."""
         batch = len(lens)
@@ -123,16 +123,10 @@ def main() -> int:
         eng = model.engine(seq_lens=room, max_seqs=batch)
         slots = eng.open(batch)
         ps = prompts(lens)
-        ids, i = [], 0
-        while i < batch:                                     # prompts of about 16k tokens per ragged step
-            j, tokens = i, 0
-            while j < batch and (j == i or tokens + lens[j] <= 16384):
-                tokens += lens[j]
-                j += 1
-            logits = eng.step(slots[i:j], ps[i:j], "last")
-            ids += ops.argmax(logits).tolist()
-            i = j
-            print(f"[bench] prefilled {i}/{batch}", file=sys.stderr, flush=True)
+        # the prompts run as the generation loop runs them: ragged steps of at most its token budget each
+        ids = ops.argmax(alice.run_prompt_steps(eng, slots, ps)).tolist()
+        print(f"[bench] prefilled {batch} prompts in {len(alice.plan_prompt_steps(lens, alice.engine.generate.MAX_STEP_TOKENS))} steps",
+              file=sys.stderr, flush=True)
         # Decode steps as the library's own generation loop runs them: the chosen ids go from the sampling kernel
         # to the next step on the device, and the host queues step n + 1 before it reads step n's ids (through a
         # pinned buffer and an event), so it is one step ahead and no further.

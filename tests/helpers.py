@@ -63,11 +63,43 @@ def model_folder(name: str, stored: str = "bfloat16", hot: float = 1.0) -> str:
     return folder
 
 
-def plain_model(folder: str, dense: bool = False):
+def write_marker_model(folder: str, raw: dict, seed: int, markers=(7, 8, 9)) -> None:
+    """A model folder with random weights, edited so that the keys of the marker tokens stand out: every query scores
+    them far above all other keys (one hidden feature that only the markers' embeddings have, read by one row of
+    every key projection; a constant feature read by the matching row of every query projection; the pair sits in
+    the rotation's slowest plane, so the score survives thousands of positions).  Among thousands of keys with nearly
+    equal weights one key more or less changes nothing that a tolerance sees; one marker more or less does."""
+    import alice_llm_amd as alice
+    from safetensors.torch import load_file, save_file
+    alice.write_random_model(folder, dict(raw), seed=seed)
+    path = os.path.join(folder, "model.safetensors")
+    t = load_file(path)
+    d, nH, nKV = raw["head_dim"], raw["num_attention_heads"], raw["num_key_value_heads"]
+    E = t["model.embed_tokens.weight"].float()
+    E[:, 0] = 0.1                       # a feature every token has
+    E[:, 1:2 + len(markers)] = 0.0
+    for n, m in enumerate(markers):
+        E[m, 1] = 0.5                   # one that only the markers have, which the keys read,
+        E[m, 2 + n] = 0.5               # and one of its own for each marker, so that their values differ
+    t["model.embed_tokens.weight"] = E.to(torch.bfloat16)
+    j = d // 2 - 1                      # the slowest plane of the rotation: rows j and j + d/2 of a head
+    for i in range(raw["num_hidden_layers"]):
+        q = t[f"model.layers.{i}.self_attn.q_proj.weight"].float()
+        k = t[f"model.layers.{i}.self_attn.k_proj.weight"].float()
+        for h in range(nH):
+            q[h * d + j, 0] += 2.0
+        for h in range(nKV):
+            k[h * d + j, 1] += 2.0
+        t[f"model.layers.{i}.self_attn.q_proj.weight"] = q.to(torch.bfloat16)
+        t[f"model.layers.{i}.self_attn.k_proj.weight"] = k.to(torch.bfloat16)
+    save_file(t, path)
+
+
+def plain_model(folder: str, dense: bool = False, device="cpu"):
     """dense: attention as one masked matrix product per head instead of key by key (the two forms are tested
     against each other); what sequences of thousands of tokens need."""
     from plain.gemma2_plain import PlainGemma2
-    return PlainGemma2.from_folder(folder, dense=dense)
+    return PlainGemma2.from_folder(folder, dense=dense, device=device)
 
 
 def random_tokens(vocab: int, n: int, seed: int):

@@ -1,10 +1,11 @@
 """Plain, slow Gemma 2 for whole sequences: the oracle of the tests.
 
 One function per formula, each written from the formula that the reference's
-single-token CPU forward computes (file:line of /root/reference in each
-docstring).  Whole sequences, dense masks, no cache, float64 by default, and
-no code shared with the package under test: it reads config.json keys and
-safetensors tensor names itself.
+single-token CPU forward computes (its file:line in each docstring).  Whole
+sequences, dense masks, no cache, float64 by default, and no code shared with
+the package under test: it reads config.json keys and safetensors tensor names
+itself.  It runs where its tensors are: on the CPU, or with `device` on a GPU
+(torch's float64 there), which is what a model of full size needs.
 
 Two deliberate differences from the reference's text, both part of this
 architecture's contract rather than of the reference's GGUF convention:
@@ -88,7 +89,7 @@ def attention_core(q, k, v, scale, cap, window):
     T, nH, d = q.shape
     nKV = k.shape[1]
     g = nH // nKV
-    out = torch.zeros(T, nH, d, dtype=q.dtype)
+    out = torch.zeros(T, nH, d, dtype=q.dtype, device=q.device)
     for p in range(T):
         start = 0 if window is None else max(0, p + 1 - window)
         for h in range(nH):
@@ -107,12 +108,12 @@ def attention_dense(q, k, v, scale, cap, window):
     T, nH, d = q.shape
     nKV = k.shape[1]
     g = nH // nKV
-    i = torch.arange(T)[:, None]
-    j = torch.arange(T)[None, :]
+    i = torch.arange(T, device=q.device)[:, None]
+    j = torch.arange(T, device=q.device)[None, :]
     allowed = j <= i
     if window is not None:
         allowed = allowed & (j >= i + 1 - window)
-    out = torch.empty(T, nH, d, dtype=q.dtype)
+    out = torch.empty(T, nH, d, dtype=q.dtype, device=q.device)
     for h in range(nH):
         s = (q[:, h, :] @ k[:, h // g, :].T) * scale
         s = softcap(s, cap)
@@ -131,9 +132,10 @@ def geglu(x, w_gate, w_up, w_down):
 class PlainGemma2:
     """Whole-sequence forward from a model folder's raw config.json and tensors."""
 
-    def __init__(self, config: dict, tensors: dict, dtype=DT, dense: bool = False):
+    def __init__(self, config: dict, tensors: dict, dtype=DT, dense: bool = False, device="cpu"):
         c = config
         self.dtype = dtype
+        self.device = torch.device(device)
         self.attention = attention_dense if dense else attention_core
         self.V = c["vocab_size"]
         self.H = c["hidden_size"]
@@ -149,10 +151,10 @@ class PlainGemma2:
         self.cap_f = c.get("final_logit_softcapping", 30.0)
         self.scale = float(c.get("query_pre_attn_scalar", self.d)) ** -0.5
         self.layer_types = c.get("layer_types")
-        self.t = {k: v.to(dtype) for k, v in tensors.items()}
+        self.t = {k: v.to(device=self.device, dtype=dtype) for k, v in tensors.items()}
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=DT, dense: bool = False):
+    def from_folder(cls, folder: str, dtype=DT, dense: bool = False, device="cpu"):
         from safetensors import safe_open
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
@@ -160,7 +162,7 @@ class PlainGemma2:
         with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
             for k in f.keys():
                 tensors[k] = f.get_tensor(k)
-        return cls(config, tensors, dtype, dense)
+        return cls(config, tensors, dtype, dense, device)
 
     def layer_window(self, i: int):
         """Even layers slide, odd layers see everything (llama3.rs:4634-4641); a config.json that lists
@@ -173,7 +175,7 @@ class PlainGemma2:
         """Row copy times sqrt(hidden) taken in f32.  llama3.rs:13686-13703."""
         E = self.t["model.embed_tokens.weight"]
         scale = float(torch.tensor(float(self.H), dtype=torch.float32).sqrt())
-        return E[torch.as_tensor(tokens, dtype=torch.long)] * scale
+        return E[torch.as_tensor(tokens, dtype=torch.long, device=self.device)] * scale
 
     def layer(self, i: int, x: torch.Tensor, positions: torch.Tensor, taps=None):
         """x + N_post_attn(Attn(N_in(x))), then x + N_post_ffn(FFN(N_pre_ffn(x))).
@@ -208,7 +210,7 @@ class PlainGemma2:
     def forward(self, tokens, taps=None) -> torch.Tensor:
         """Logits [T, V] of one whole sequence.  llama3.rs:13632-14614."""
         T = len(tokens)
-        positions = torch.arange(T)
+        positions = torch.arange(T, device=self.device)
         x = self.embed(tokens)
         for i in range(self.L):
             x = self.layer(i, x, positions, taps)

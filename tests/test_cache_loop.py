@@ -154,9 +154,11 @@ class FakeEngine:
     def step(self, slots, tokens, want):
         self.cache.reserve(slots, [len(t) for t in tokens]); self.cache.commit(slots, [len(t) for t in tokens])
         self.steps.append((list(slots), [len(t) for t in tokens]))
-        out = torch.zeros(len(slots), self.V)
-        for i, t in enumerate(tokens):
-            out[i, (t[-1] + 1) % self.V] = 1.0
+        rows = [i for i in range(len(slots)) if want == "last" or (not isinstance(want, str) and want[i])]
+        assert want == "last" or all(want[i] == [len(tokens[i]) - 1] for i in rows)    # the loop asks for last rows only
+        out = torch.zeros(len(rows), self.V)
+        for r, i in enumerate(rows):
+            out[r, (tokens[i][-1] + 1) % self.V] = 1.0
         return out
 
 
@@ -173,6 +175,56 @@ def test_plan_batches():
     assert plan_batches([60, 60], [5, 5], max_batch=None, capacity_tokens=128, max_slots=8, page=64) == [[0, 1]]
     with pytest.raises(ValueError, match="request 1"):
         plan_batches([5, 300], [8, 8], max_batch=4, capacity_tokens=256, max_slots=4, page=64)
+
+
+def test_plan_prompt_steps():
+    from alice_llm_amd.engine.generate import plan_prompt_steps
+    assert plan_prompt_steps([5, 12, 17], None) == [[(0, 0, 5), (1, 0, 12), (2, 0, 17)]]
+    assert plan_prompt_steps([5, 12, 17], 100) == [[(0, 0, 5), (1, 0, 12), (2, 0, 17)]]
+    # every step but the last is full; a prompt goes on where the step before left it
+    assert plan_prompt_steps([5, 12, 17], 7) == [[(0, 0, 5), (1, 0, 2)], [(1, 2, 7)], [(1, 9, 3), (2, 0, 4)], [(2, 4, 7)], [(2, 11, 6)]]
+    assert plan_prompt_steps([3, 3], 3) == [[(0, 0, 3)], [(1, 0, 3)]]
+    assert plan_prompt_steps([4], 1) == [[(0, i, 1)] for i in range(4)]
+    for lens, budget in (([6000] * 8, 16384), ([1, 70, 64, 129, 2], 64), ([9], 2)):
+        steps = plan_prompt_steps(lens, budget)
+        assert all(sum(n for _, _, n in st) == budget for st in steps[:-1]) and 0 < sum(n for _, _, n in steps[-1]) <= budget
+        assert all(len({i for i, _, _ in st}) == len(st) for st in steps)              # a sequence once per step
+        at = [0] * len(lens)
+        for st in steps:
+            for i, a, n in st:
+                assert a == at[i] and n > 0
+                at[i] += n
+        assert at == lens
+    with pytest.raises(ValueError):
+        plan_prompt_steps([3], 0)
+
+
+def test_the_loop_cuts_prompts_into_steps_of_its_budget():
+    """Prompts that hold more tokens than a step's budget run in several steps, a long one in pieces; what the loop
+    decides afterwards is what it decides with everything in one step."""
+    prompts = [[1, 2, 3, 4, 5, 6, 7, 8, 9], [7], [4, 5, 6, 7, 8], [12, 13]]
+    caps = [3, 4, 2, 5]
+    runs = {}
+    for budget in (None, 64, 7, 4, 1):
+        eng = FakeEngineAhead(n_slots=4)
+        res = Generator(eng, stop_token_ids=[], sampler=argmax_sampler, max_step_tokens=budget).run(prompts, caps)
+        runs[budget] = [r.tokens for r in res]
+        n_prompt_steps = len(plan_prompt_steps_of(budget, prompts))
+        assert n_prompt_steps == {None: 1, 64: 1, 7: 3, 4: 5, 1: 17}[budget]
+        fed = [0] * 4
+        for sl, ns in eng.steps[:n_prompt_steps]:
+            assert sum(ns) <= (budget or 17)
+            for s_, n in zip(sl, ns):
+                fed[eng.opened.index(s_)] += n
+        assert fed == [9, 1, 5, 2]
+        assert eng.cache.slots.n_free() == 4
+        eng.cache.check_consistent()
+    assert all(r == runs[None] for r in runs.values()) and runs[None] == [[10, 11, 12], [8, 9, 10, 11], [9, 10], [14, 15, 0, 1, 2]]
+
+
+def plan_prompt_steps_of(budget, prompts):
+    from alice_llm_amd.engine.generate import plan_prompt_steps
+    return plan_prompt_steps([len(p) for p in prompts], budget)
 
 
 def test_requests_that_would_outgrow_the_positions():

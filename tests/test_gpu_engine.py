@@ -134,18 +134,47 @@ def plain_model_without_caps(plain):
     return p
 
 
-def test_stored_float32_stays_float32_and_agrees():
-    model, plain = setup("tiny-b", "float32", stored="float32")
-    lin = model.lm.layers[0].mixer.qkv
-    assert lin.weight.dtype == torch.float32 and model.lm.layers[0].norms["pre_mixer"].weight.dtype == torch.float32
-    mb, _ = setup("tiny-b", "bfloat16", stored="float32")
-    assert mb.lm.layers[0].mixer.qkv.weight.dtype == torch.float32                # not narrowed behind the user's back
-    toks = random_tokens(plain.V, 33, 14)
+def linears_of(model):
+    from alice_llm_amd.parts.linear import Linear
+    return [(prefix + k, v) for prefix, part in model.lm.named_parts() for k, v in vars(part).items() if isinstance(v, Linear)]
+
+
+def plain_with_rounded_matrices(folder, dense=False):
+    """The plain implementation fed with the folder's tensors, its matrices rounded to bfloat16 (norm weights as stored)."""
+    import json, os
+    from safetensors.torch import load_file
+    from plain.gemma2_plain import PlainGemma2
+    with open(os.path.join(folder, "config.json")) as f:
+        config = json.load(f)
+    tensors = {k: (v.to(torch.bfloat16) if v.dim() == 2 else v) for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    return PlainGemma2(config, tensors, dense=dense)
+
+
+@pytest.mark.parametrize("name", ["tiny-b", "tiny-c"])
+def test_stored_float32_is_rounded_once_on_the_bfloat16_path(name):
+    """A folder stored in 32-bit: the 32-bit path keeps it, the bfloat16 path rounds every matrix to bfloat16 at load
+    and runs it on the matrix-core kernels like a folder stored in bfloat16 (norm weights stay 32-bit); the run
+    that keeps stored dtypes leaves the matrices 32-bit."""
+    from alice_llm_amd.hip import ops
+    folder = model_folder(name, "float32")
+    model, plain = setup(name, "float32", stored="float32")
+    assert all(l.weight.dtype == torch.float32 for _, l in linears_of(model))
+    assert model.lm.layers[0].norms["pre_mixer"].weight.dtype == torch.float32
+    mb, _ = setup(name, "bfloat16", stored="float32")
+    assert len(linears_of(mb)) >= 4 * len(mb.lm.layers) + 1
+    for where, l in linears_of(mb):
+        assert l.weight.dtype == torch.bfloat16 and l.layout == ops.LAYOUT_FRAG16, where
+    assert mb.lm.layers[0].norms["pre_mixer"].weight.dtype == torch.float32
+    mk = alice.load(folder, dtype="bfloat16", keep_stored_dtype=True)
+    assert all(l.weight.dtype == torch.float32 and l.layout == ops.LAYOUT_ROW for _, l in linears_of(mk))
+    toks = random_tokens(plain.V, 133, 14)
     ref = plain.forward(toks)
-    for m, d in ((model, "float32"), (mb, "bfloat16")):
-        eng = m.engine(max_tokens=64)
+    rounded = plain_with_rounded_matrices(folder).forward(toks)
+    for m, d, r in ((model, "float32", ref), (mb, "bfloat16", rounded), (mk, "bfloat16", ref)):
+        eng = m.engine(max_tokens=256)
         s = eng.open(1)
-        assert max_err(eng.step(s, [toks], "all"), ref) < tol(d, ref)
+        got = [eng.step(s, [toks[:101]], "all")] + [eng.step(s, [[t]], "last") for t in toks[101:]]
+        assert max_err(torch.cat(got), r) < tol(d, r), d
 
 
 def test_step_argument_errors():

@@ -45,6 +45,66 @@ def test_greedy_generation_matches_plain(name, lens, steps):
             seq.append(tok)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompts_cut_into_steps_of_a_token_budget_give_the_same_tokens(dtype):
+    """The loop runs a batch's prompts in ragged steps of at most max_step_tokens tokens: with budgets of 7 and 64
+    (pieces that start and end inside pages and inside the window of 6, a piece of one token, a request that a step
+    leaves out) and with none, greedy generation gives the same tokens, the plain implementation's."""
+    folder = model_folder("tiny-b", "bfloat16")
+    plain = plain_model(folder)
+    prompts = [random_tokens(plain.V, n, 50 + i) for i, n in enumerate((3, 71, 14, 129, 1, 64))]
+    model = alice.load(folder, dtype=dtype)
+    steps_of = lambda budget: alice.plan_prompt_steps([len(p) for p in prompts], budget)
+    assert [len(steps_of(b)) for b in (None, 64, 7)] == [1, 5, 41]
+    assert any(n == 1 for st in steps_of(7) for _, _, n in st) and any(len(st) == 1 for st in steps_of(7))
+    runs = {b: [r.tokens for r in model.generate(prompts, max_new_tokens=6, stop_token_ids=[], max_step_tokens=b)]
+            for b in (None, 64, 7)}
+    if dtype == "float32":
+        assert runs[None] == [plain.greedy(p, 6) for p in prompts]
+        assert runs[64] == runs[None] and runs[7] == runs[None]
+    else:
+        for b, run in runs.items():           # bfloat16: every chosen token within rounding of the plain maximum
+            for p, toks in zip(prompts, run):
+                seq = list(p)
+                for tok in toks:
+                    lg = plain.forward(seq)[-1]
+                    assert float(lg.max() - lg[tok]) < 0.03, b
+                    seq.append(tok)
+    # the logits at the prompts' last tokens, through the loop's own prompt steps, against the plain implementation
+    eng = model.engine(seq_lens=[len(p) for p in prompts])
+    for b in (None, 64, 7):
+        slots = eng.open(len(prompts))
+        got = alice.run_prompt_steps(eng, slots, prompts, b)
+        eng.close(slots)
+        ref = torch.stack([plain.forward(p)[-1] for p in prompts])
+        assert (got.double().cpu() - ref).abs().max() < (2e-5 if dtype == "float32" else 3e-2) * max(1.0, float(ref.abs().max())), b
+    eng.cache.check_consistent()
+
+
+def test_generate_keeps_its_engine_between_calls():
+    """Model.generate without an engine makes one and keeps it: a second call of the same shapes runs on the same
+    cache and captures nothing new; a call that does not fit gets a larger engine."""
+    folder = model_folder("tiny-c", "bfloat16")
+    plain = plain_model(folder)
+    model = alice.load(folder, dtype="bfloat16")
+    prompts = [random_tokens(plain.V, n, 60 + i) for i, n in enumerate((9, 30, 17))]
+    a = model.generate(prompts, max_new_tokens=8, stop_token_ids=[])
+    eng = model._kept_engine
+    assert eng is not None and eng.use_graphs and len(eng._graphs) >= 1
+    graphs = dict(eng._graphs)
+    prompt_graphs = dict(eng._prompt_graphs)
+    b = model.generate(prompts, max_new_tokens=8, stop_token_ids=[])
+    assert model._kept_engine is eng and [r.tokens for r in a] == [r.tokens for r in b]
+    assert eng._graphs.keys() == graphs.keys() and all(eng._graphs[k] is g for k, g in graphs.items())
+    c = model.generate(prompts[:2], max_new_tokens=5, stop_token_ids=[])            # smaller: fits
+    assert model._kept_engine is eng and [len(r.tokens) for r in c] == [5, 5]
+    d = model.generate(prompts + prompts, max_new_tokens=8, stop_token_ids=[])      # more sequences at once: a new engine
+    assert model._kept_engine is not eng and [len(r.tokens) for r in d] == [8] * 6
+    assert model._kept_engine.cache.slots.n_free() == 6
+    model.release_engine()
+    assert model._kept_engine is None
+
+
 def test_temperature_sampling_is_reproducible_and_batch_independent():
     folder = model_folder("tiny-b", "bfloat16")
     plain = plain_model(folder)
@@ -122,6 +182,13 @@ def test_command_line(tmp_path):
         assert d["token"] == seq[d["position"] + 1] == d["top5"][0][0]
         assert [t for t, _ in d["top5"]] == top.indices.tolist()
         assert max(abs(v - float(w)) for (_, v), w in zip(d["top5"], top.values)) < 2e-5
+    # --dump-logits FILE: the same lines in a file, for every generated position
+    path = tmp_path / "dump.jsonl"
+    proc = subprocess.run(cmd[:-2] + ["--dump-logits", str(path)], capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert not [l for l in proc.stderr.splitlines() if l.startswith("{")]
+    filed = [json.loads(l) for l in path.read_text().splitlines()]
+    assert len(filed) == 10 and [d for d in filed if d["position"] in dict([(0, (3, 4)), (1, (1, 2))])[d["request"]]] == dumps
 
 
 def test_logits_dump_follows_the_sampler_of_the_run():
@@ -131,9 +198,8 @@ def test_logits_dump_follows_the_sampler_of_the_run():
     from alice_llm_amd.generate import _logits_dumper
     import contextlib, io, json
     err = io.StringIO()
-    with contextlib.redirect_stderr(err):
-        res = model.generate([[3, 4, 5], [9]], max_new_tokens=6, temperature=1.5, seed=3, stop_token_ids=[],
-                             observer=_logits_dumper(4))
+    res = model.generate([[3, 4, 5], [9]], max_new_tokens=6, temperature=1.5, seed=3, stop_token_ids=[],
+                         observer=_logits_dumper(4, err))
     dumps = [json.loads(l) for l in err.getvalue().splitlines()]
     assert len(dumps) == 8
     for r in (0, 1):

@@ -4,9 +4,7 @@ pieces of a prompt on a long cached prefix, decode batches of 16 to 130 through 
 
 Random N(0, 0.02) weights would hide a key that is read one place too far: among thousands of keys with nearly
 equal weights one more or less changes nothing that a tolerance sees.  The models here therefore carry a marker:
-tokens whose keys every query scores far above all others (one hidden feature that only the markers' embeddings
-have, read by one row of every key projection; a constant feature read by the matching row of every query
-projection; the pair sits in the rotation's slowest plane, so the score survives thousands of positions).  Markers
+tokens whose keys every query scores far above all others (helpers.write_marker_model).  Markers
 are placed so that the window's edge passes over them in a prompt piece, in single-token steps, and in a piece
 that follows after pages were given back; the tests assert that the plain implementation with a window one key
 longer differs there by far more than the tolerance, so a kernel that is off by one cannot pass.
@@ -18,7 +16,7 @@ import pytest
 import torch
 
 import alice_llm_amd as alice
-from helpers import TOL, max_err, plain_model, random_tokens
+from helpers import TOL, max_err, plain_model, random_tokens, write_marker_model
 
 pytestmark = pytest.mark.gpu
 _TMP = tempfile.TemporaryDirectory(prefix="alice_long_")
@@ -43,31 +41,9 @@ def marker_model(name):
     """(folder, plain model, tokens, layout): a random model edited so that the marker's key stands out."""
     if name in _CASES:
         return _CASES[name]
-    from safetensors.torch import load_file, save_file
     raw = dict(LONG[name])
     folder = os.path.join(_TMP.name, name)
-    alice.write_random_model(folder, raw, seed=11)
-    path = os.path.join(folder, "model.safetensors")
-    t = load_file(path)
-    d, nH, nKV = raw["head_dim"], raw["num_attention_heads"], raw["num_key_value_heads"]
-    E = t["model.embed_tokens.weight"].float()
-    E[:, 0] = 0.1                       # a feature every token has
-    E[:, 1:2 + len(MARKERS)] = 0.0
-    for n, m in enumerate(MARKERS):
-        E[m, 1] = 0.5                   # one that only the markers have, which the keys read,
-        E[m, 2 + n] = 0.5               # and one of its own for each marker, so that their values differ
-    t["model.embed_tokens.weight"] = E.to(torch.bfloat16)
-    j = d // 2 - 1                      # the slowest plane of the rotation: rows j and j + d/2 of a head
-    for i in range(raw["num_hidden_layers"]):
-        q = t[f"model.layers.{i}.self_attn.q_proj.weight"].float()
-        k = t[f"model.layers.{i}.self_attn.k_proj.weight"].float()
-        for h in range(nH):
-            q[h * d + j, 0] += 2.0
-        for h in range(nKV):
-            k[h * d + j, 1] += 2.0
-        t[f"model.layers.{i}.self_attn.q_proj.weight"] = q.to(torch.bfloat16)
-        t[f"model.layers.{i}.self_attn.k_proj.weight"] = k.to(torch.bfloat16)
-    save_file(t, path)
+    write_marker_model(folder, raw, seed=11, markers=MARKERS)
     W = raw["sliding_window"]
     # the sequence: a prompt, a second piece that crosses the window, single tokens, a third piece that starts after
     # pages were given back, single tokens again

@@ -397,10 +397,13 @@ class ToyScanConfig(ToyConfig):
 
 
 def toy_scan_plain(model, tokens):
+    E = model.lm.embedding.table.weight.double().cpu()
+    return _toy_scan_plain_from(model, E[torch.tensor(tokens)], E)
+
+
+def _toy_scan_plain_from(model, x, E):
     lm = model.lm
-    E = lm.embedding.table.weight.double().cpu()
-    x = E[torch.tensor(tokens)]
-    T = len(tokens)
+    T = x.shape[0]
     rms = lambda v, n: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + n.eps) * (n.weight_offset + n.weight.double().cpu())
     for layer in lm.layers:
         h = rms(x, layer.norms["pre_mixer"])
@@ -464,6 +467,227 @@ def test_toy_mixer_with_two_state_tensors_runs_in_captured_steps():
             assert (got[graph][i].double().cpu() - refs[i]).abs().max() < 2e-5 * max(1.0, float(refs[i].abs().max())), (again, i)
             assert (got[graph][i] - got[eager][i]).abs().max() < 1e-5
     assert len(graph._graphs) >= 3                               # batches of 3 (a bucket of 4), 2 and 1
+
+
+class ToyTailScanDeviceMixer(ToyTailScanMixer):
+    """The same mixer with its steps of several tokens on the device as well: a scan over the step's longest
+    piece whose rows come from ctx.cu_seqlens, with sequences that have ended masked out.  It therefore declares
+    graph_safe_prompts, and short prompt steps of its model are recorded into HIP graphs like the built-in parts'."""
+    graph_safe_prompts = True
+
+    def forward(self, x, ctx, cache):
+        if ctx.is_decode:
+            return super().forward(x, ctx, cache)
+        u = x.float() @ self.w["in.weight"].T
+        tail, acc = cache.state["tail"], cache.state["sum"]
+        T = u.shape[0]
+        idx, cu = ctx.slots.long(), ctx.cu_seqlens.long()
+        held = tail.index_select(0, idx)
+        t2, t1, s = held[:, 0], held[:, 1], acc.index_select(0, idx)
+        u_pad = torch.cat([u, torch.zeros_like(u[:1])])
+        out = torch.zeros_like(u_pad)                            # row T takes what ended sequences write
+        dump = torch.full_like(cu[:-1], T)
+        for t in range(ctx.max_new):                             # a host constant of the (captured) step
+            rows = cu[:-1] + t
+            live = rows < cu[1:]
+            rows = torch.where(live, rows, dump)
+            ut = u_pad.index_select(0, rows)
+            lv = live[:, None]
+            s = torch.where(lv, self.decay * s + ut + 0.5 * t1 + 0.25 * t2, s)
+            t2, t1 = torch.where(lv, t1, t2), torch.where(lv, ut, t1)
+            out.index_copy_(0, rows, s)
+        acc.index_copy_(0, idx, s)
+        tail.index_copy_(0, idx, torch.stack([t2, t1], dim=1))
+        return (out[:T] @ self.w["out.weight"].T).contiguous()
+
+
+class ToyLearnedPositions(alice.parts.embedding.Embedding):
+    """An embedding that adds a learned row per position: it needs the step's positions, which it finds in ctx."""
+
+    def __init__(self, precision, *, vocab_size, dim, max_positions, scale=1.0):
+        super().__init__(precision, vocab_size=vocab_size, dim=dim, scale=scale)
+        self.P = max_positions
+
+    def param_specs(self):
+        return {**super().param_specs(), "positions.weight": ParamSpec((self.P, self.dim), 0.3)}
+
+    def assign(self, name, t):
+        if name == "positions.weight":
+            self.pos = t.float()
+        else:
+            super().assign(name, t)
+
+    def forward(self, ctx):
+        return super().forward(ctx) + self.pos.index_select(0, ctx.positions.long())
+
+
+class ToyScanDeviceConfig(ToyScanConfig):
+    def plan(self):
+        import dataclasses
+        plan = super().plan()
+        swap = lambda m: PartSpec("toy_tail_scan_device", m.args, m.name) if m.kind == "toy_tail_scan" else m
+        layers = tuple(dataclasses.replace(l, mixer=swap(l.mixer)) for l in plan.layers)
+        emb = PartSpec("toy_learned_positions", {"vocab_size": plan.vocab_size, "dim": plan.hidden_size, "max_positions": 256}, "emb")
+        return dataclasses.replace(plan, layers=layers, embedding=emb)
+
+
+def test_toy_embedding_reads_positions_and_stateful_prompt_steps_are_captured():
+    """An embedding that needs the step's positions and a stateful mixer that advances its state on the device in
+    steps of several tokens: registered from here; the engine then records short prompt steps of this model too,
+    and a recorded step gives what the eager one and the plain replica give."""
+    from alice_llm_amd.parts import EMBEDDINGS
+    MIXERS.register("toy_tail_scan", ToyTailScanMixer)
+    MIXERS.register("toy_tail_scan_device", ToyTailScanDeviceMixer)
+    FEED_FORWARDS.register("toy_graph_mlp", ToyGraphMLP)
+    EMBEDDINGS.register("toy_learned_positions", ToyLearnedPositions)
+    alice.register_architecture("ToyScanDeviceForCausalLM", ToyScanDeviceConfig)
+    alice.register_architecture("ToyScanForCausalLM", ToyScanConfig)
+    raw = {"architectures": ["ToyScanDeviceForCausalLM"], "width": 48, "vocab": 83, "state": 20}
+    model = alice.Model.random(raw, seed=8, dtype="float32", stored_dtype=torch.float32)
+    assert "emb.positions.weight" in model.lm.param_specs()
+    graph = model.engine(max_tokens=64 * 6, max_seqs=4)
+    eager = model.engine(max_tokens=64 * 6, max_seqs=4, use_graphs=False)
+    assert graph.capture_prompts and not eager.capture_prompts
+    host_only = alice.Model.random(dict(raw, architectures=["ToyScanForCausalLM"]), seed=8, dtype="float32", stored_dtype=torch.float32)
+    assert not host_only.engine(max_tokens=64).capture_prompts        # its prompts loop on the host: not recorded
+
+    def plain(tokens):                                                # the replica of the scan toy plus the position rows
+        lm = model.lm
+        E, Ppos = lm.embedding.table.weight.double().cpu(), lm.embedding.pos.double().cpu()
+        return _toy_scan_plain_from(model, E[torch.tensor(tokens)] + Ppos[:len(tokens)], E)
+
+    g = torch.Generator().manual_seed(10)
+    seqs = [torch.randint(0, 83, (n,), generator=g).tolist() for n in (29, 17, 23)]
+    refs = [plain(t) for t in seqs]
+    for again in range(3):                                            # the third pass replays what the second recorded
+        got = {}
+        for eng in (graph, eager):
+            slots = eng.open(3)
+            rows = {i: [] for i in range(3)}
+            at = [0, 0, 0]
+            for piece in ((5, 2, 7), (6, 6, 1), (3, 4, 9)):           # pieces of prompts, last rows wanted: 14, 13, 16 tokens
+                lg = eng.step(slots, [seqs[i][at[i]:at[i] + n] for i, n in enumerate(piece)], "last")
+                for i, n in enumerate(piece):
+                    at[i] += n
+                    rows[i].append((at[i] - 1, lg[i].clone()))
+            live = [0, 1, 2]
+            while live:
+                lg = eng.step([slots[i] for i in live], [[seqs[i][at[i]]] for i in live], "last")
+                for r, i in enumerate(live):
+                    rows[i].append((at[i], lg[r].clone()))
+                    at[i] += 1
+                done = [i for i in live if at[i] >= len(seqs[i])]
+                eng.close([slots[i] for i in done])
+                live = [i for i in live if i not in done]
+            got[eng] = rows
+            eng.cache.check_consistent()
+        for i in range(3):
+            for (p, a), (p2, b) in zip(got[graph][i], got[eager][i]):
+                assert p == p2 and (a - b).abs().max() < 1e-5, (again, i, p)
+                assert (a.double().cpu() - refs[i][p]).abs().max() < 2e-5 * max(1.0, float(refs[i].abs().max())), (again, i, p)
+    assert len(graph._prompt_graphs) >= 2                             # token counts 14, 13 and 16 round to 16: two shapes (with and without padding)
+
+
+class ToyF32KeyMixer(Part):
+    """One head of plain causal attention, in torch, that keeps its keys and values in 32-bit whatever the run's
+    activation dtype is: it says so in its KVNeed, and the cache gives its layers pages of their own in that dtype."""
+
+    def __init__(self, precision, positions, *, hidden_size, head_dim):
+        self.H, self.d = hidden_size, head_dim
+        self.w = {}
+
+    def param_specs(self):
+        return {f"{n}.weight": ParamSpec((self.d, self.H), 0.2) for n in "qkv"} | {"o.weight": ParamSpec((self.H, self.d), 0.2)}
+
+    def assign(self, name, t):
+        self.w[name] = t.float()
+
+    def cache_need(self):
+        from alice_llm_amd.parts import KVNeed
+        return CacheNeed(kv=KVNeed(1, self.d, dtype=torch.float32))
+
+    def forward(self, x, ctx, cache):
+        assert cache.k.dtype == torch.float32 and cache.v.dtype == torch.float32
+        x = x.float()
+        q, k, v = (x @ self.w[f"{n}.weight"].T for n in "qkv")
+        P_ = cache.k.shape[2]
+        pos, seq = ctx.positions.long(), ctx.seq_of_token.long()
+        page = cache.block_table.long()[seq, pos // P_]
+        cache.k[page, 0, pos % P_] = k
+        cache.v[page, 0, pos % P_] = v
+        out = torch.empty_like(q)
+        row = 0
+        for b, (start, n) in enumerate(zip(ctx.start_lens, ctx.new_lens)):
+            pages = cache.block_table[b, :-(-(start + n) // P_)].long()
+            keys, vals = cache.k[pages, 0].reshape(-1, self.d)[:start + n], cache.v[pages, 0].reshape(-1, self.d)[:start + n]
+            sc = (q[row:row + n] @ keys.T) * self.d ** -0.5
+            mask = torch.arange(start + n, device=x.device)[None, :] > (start + torch.arange(n, device=x.device))[:, None]
+            out[row:row + n] = torch.softmax(sc.masked_fill(mask, float("-inf")), -1) @ vals
+            row += n
+        return (out @ self.w["o.weight"].T).contiguous()
+
+
+class ToyMixedKeysConfig(ToyConfig):
+    def plan(self):
+        H, V = self.d["width"], self.d["vocab"]
+        norm = lambda name: PartSpec("rmsnorm", {"dim": H, "eps": 1e-5, "weight_offset": 0.0}, name)
+        mixers = [PartSpec("toy_f32_keys", {"hidden_size": H, "head_dim": 24}, "mix"),
+                  PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16, "scale": 0.25,
+                                         "position": "rope"}, "attn")]
+        layers = [LayerPlan(block="prenorm", mixer=m, feed_forward=PartSpec("toy_mlp", {"hidden_size": H}, "ff"),
+                            norms={"pre_mixer": norm("n1"), "pre_ff": norm("n2")}, prefix=f"blocks.{i}.") for i, m in enumerate(mixers)]
+        return ModelPlan(vocab_size=V, hidden_size=H, max_positions=256,
+                         embedding=PartSpec("embedding", {"vocab_size": V, "dim": H, "scale": 1.0}, "emb"),
+                         positions={"rope": PartSpec("rope", {"dim": 16, "theta": 100.0, "max_positions": 256})},
+                         layers=tuple(layers), schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+                         final_norm=norm("final"), head=PartSpec("lm_head", {"vocab_size": V, "dim": H, "tied_to": "emb"}, "head"))
+
+
+def test_toy_mixer_keeps_32_bit_keys_under_bfloat16_activations():
+    """A mixer names the dtype of its pages in its KVNeed: in a bfloat16 run its layers get 32-bit pages of their
+    own beside the built-in attention's bfloat16 pages, and what they hold was never rounded."""
+    MIXERS.register("toy_f32_keys", ToyF32KeyMixer)
+    FEED_FORWARDS.register("toy_mlp", ToyMLP)
+    alice.register_architecture("ToyMixedKeysForCausalLM", ToyMixedKeysConfig)
+    raw = {"architectures": ["ToyMixedKeysForCausalLM"], "width": 64, "vocab": 71}
+    model = alice.Model.random(raw, seed=9, dtype="bfloat16")
+    eng = model.engine(max_tokens=256, max_seqs=2)
+    assert sorted((g.layers, g.k.dtype, g.need.head_dim) for g in eng.cache.groups) == \
+        [([0], torch.float32, 24), ([1], torch.bfloat16, 16)]
+    assert not eng.use_graphs                                    # the toy loops on the host
+    seqs = [[5, 9, 3, 70, 1, 22, 8, 8, 41, 60, 2, 13, 44, 6], [7, 7, 30, 12]]
+    slots = eng.open(2)
+    whole = eng.step(slots, seqs, "all")
+    # the first layer's pages hold its keys to the last bit: x W_k in 32-bit of the normed embedding rows
+    lm, m = model.lm, model.lm.layers[0].mixer
+    from types import SimpleNamespace
+    toks = torch.tensor(seqs[0] + seqs[1], dtype=torch.int32, device=DEV)      # the step's rows, so that the product is the same call
+    x0 = lm.embedding.forward(SimpleNamespace(tokens=toks))
+    h = lm.layers[0].norms["pre_mixer"].forward(x0, torch.bfloat16)
+    page = eng.cache.groups[[g.layers for g in eng.cache.groups].index([0])]
+    held = page.k[0, page.table(slots[0])[0], 0, :len(seqs[0])]
+    assert torch.equal(held, (h.float() @ m.w["k.weight"].T)[:len(seqs[0])]) and not torch.equal(held, held.bfloat16().float())
+    eng.close(slots)
+    # cut into steps, the shorter request ending earlier: the same logits within bfloat16 rounding
+    slots = eng.open(2)
+    first = eng.step(slots, [s[:3] for s in seqs], "all")
+    outs = {0: [first[:3]], 1: [first[3:]]}
+    for i in range(3, len(seqs[0])):
+        live = [b for b in (0, 1) if i < len(seqs[b])]
+        lg = eng.step([slots[b] for b in live], [[seqs[b][i]] for b in live], "last")
+        for row, b in enumerate(live):
+            outs[b].append(lg[row:row + 1])
+        if i + 1 == len(seqs[1]):
+            eng.close([slots[1]])
+    eng.close([slots[0]])
+    cut = torch.cat([torch.cat(outs[0]), torch.cat(outs[1])])
+    assert (cut - whole).abs().max() < 3e-2 * max(1.0, float(whole.abs().max()))
+    eng.cache.check_consistent()
+    # two runs that share a cache must agree on its dtype
+    import dataclasses
+    bad = dataclasses.replace(model.lm.plan, schedule=(ScheduleEntry(0), ScheduleEntry(1, cache_from=0)))
+    with pytest.raises(ValueError, match="cannot read the cache"):
+        CausalLM(bad, "bfloat16", DEV)
 
 
 # ------------------------------------------------------------------ a second toy: routing and another position encoding
@@ -625,7 +849,8 @@ def test_embedding_and_tied_head_parts(prec):
     emb.assign("weight", E)
     emb.finalize(); head.finalize(); head.tie(emb)
     tok = torch.tensor([0, 202, 17, 17], dtype=torch.int32, device=DEV)
-    x = emb.forward(tok)
+    from types import SimpleNamespace
+    x = emb.forward(SimpleNamespace(tokens=tok))
     assert x.dtype == torch.float32 and (x.double() - E.double()[tok.long()] * 2.5).abs().max() < 1e-6
     n = rnd(5, H, seed=31, dtype=p.act)
     logits = head.forward(n)
