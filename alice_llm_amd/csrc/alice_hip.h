@@ -112,15 +112,18 @@ int alice_linear_parts(const float* parts, int splits, int nH, int d, const void
 int alice_argmax_chunks(int B, int V);
 int alice_argmax(const float* logits, int* out, float* work_v, int* work_i, int B, int V, hipStream_t stream);
 // The same argmax with no workspace argument and no allocation of any kind: the chunk maxima go to a device
-// array inside the library (ALICE_ARGMAX_STATIC_MAX_PAIRS pairs of a float and an int, 32 KB, which every GPU
-// that the library runs on holds until the process ends).  It has no counterpart in the reference; it is for
+// array inside the library (ALICE_ARGMAX_STATIC_MAX_PAIRS pairs of a float and an int, 4 KB, which every GPU
+// that the library runs on holds until the process ends; it is the most that the chunk rule of
+// alice_argmax_chunks ever asks for, ALICE_ARGMAX_MAX_PARTIALS, so no number of rows or vocabulary is too large).  It has no counterpart in the reference; it is for
 // callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
 // hipMalloc.  It calls no hipMalloc, hipFree or allocating library routine; the caller passes logits and out
-// as for alice_argmax.  Rows x chunks (alice_argmax_chunks) beyond the maximum are refused with an error.  All
+// as for alice_argmax.  Rows x chunks beyond the maximum are refused with an error (a check that the chunk rule
+// keeps from firing; missing pointers and bad sizes are refused the same way).  All
 // calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads) race;
 // calls on one stream follow each other and are safe.  alice_argmax_static_init() resolves the array's address
 // for the current device ahead of the first call (the first call on a device does it otherwise).
-#define ALICE_ARGMAX_STATIC_MAX_PAIRS 4096
+#define ALICE_ARGMAX_MAX_PARTIALS 512
+#define ALICE_ARGMAX_STATIC_MAX_PAIRS ALICE_ARGMAX_MAX_PARTIALS
 int alice_argmax_static_init();
 int alice_argmax_static(const float* logits, int* out, int B, int V, hipStream_t stream);
 // temperature -> top-k (0: off) -> top-p (>= 1: off) -> softmax -> first index whose cumulative

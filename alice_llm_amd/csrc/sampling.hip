@@ -657,10 +657,11 @@ __host__ inline void sample_shape(int B, int V, int* chunks, int* tiles, int* pe
 
 }  // namespace
 
-// How many chunks a row is cut into; the workspace holds B * chunks floats and as many ints.
+// How many chunks a row is cut into; the workspace holds B * chunks floats and as many ints, which is never more
+// than ALICE_ARGMAX_MAX_PARTIALS of each: the bound that sizes the static workspace of alice_argmax_static.
 extern "C" int alice_argmax_chunks(int B, int V) {
   if (V < 16384) return 1;
-  int c = 512 / (B > 0 ? B : 1);
+  int c = ALICE_ARGMAX_MAX_PARTIALS / (B > 0 ? B : 1);
   if (c > V / 8192) c = V / 8192;
   return c < 2 ? 1 : (c > 64 ? 64 : c);
 }
@@ -688,6 +689,8 @@ extern "C" int alice_argmax(const float* logits, int* out, float* work_v, int* w
 // allocates.  Every GPU holds its own copy of the array at its own address, which the host learns once per
 // device from hipGetSymbolAddress (in host code the array's name is only a stand-in, not a device address).
 // Nothing in the array has to start at zero: stage one writes every pair that stage two reads.
+static_assert(ALICE_ARGMAX_STATIC_MAX_PAIRS >= ALICE_ARGMAX_MAX_PARTIALS,
+              "the static workspace must hold what the chunk rule can ask for");
 static __device__ __align__(256) unsigned char argmax_scratch[ALICE_ARGMAX_STATIC_MAX_PAIRS * 8];
 
 namespace {

@@ -241,6 +241,52 @@ def test_captured_decode_steps_match_eager_on_every_replay(name, dtype):
     graph.cache.check_consistent()
 
 
+def test_captured_prompt_pieces_on_a_long_prefix_past_the_window():
+    """Recorded prompt steps in their second context bucket (keys up to 1,024) with the matrix-core kernels: pieces
+    of 2 to 256 tokens on cached prefixes of more than 512 tokens, far enough past the window of 80 that the
+    sliding layers' first pages were given back and their block-table entries point at the spare page.  The list of
+    requests runs three times (seen once, recorded, replayed); every step against the eager engine and the plain
+    implementation, the replay bit for bit against the recording pass."""
+    model, plain = setup("tiny-c", "bfloat16")
+    eager = model.engine(max_tokens=64 * 40, max_seqs=4, use_graphs=False)
+    graph = model.engine(max_tokens=64 * 40, max_seqs=4, use_graphs=True)
+    assert graph.capture_prompts
+    win = [g for g in graph.cache.groups if g.need.window is not None][0]
+    # (prefix lengths, then the pieces' lengths one step after another)
+    rounds = [((530,), [(2,), (256,), (17,)]), ((600, 520), [(100, 30), (7, 9)]), ((700,), [(64,), (64,), (3,)]),
+              ((515, 640, 580), [(5, 1, 60)])]
+    recorded = {}
+    for again in range(3):
+        for r, (prefix, pieces) in enumerate(rounds):
+            total = [n + sum(p[i] for p in pieces) for i, n in enumerate(prefix)]
+            full = [random_tokens(plain.V, n, 700 + 10 * r + i) for i, n in enumerate(total)]
+            refs = [plain.forward(s) for s in full]
+            se, sg = eager.open(len(prefix)), graph.open(len(prefix))
+            feed = [s[:n] for s, n in zip(full, prefix)]
+            eager.step(se, feed, "none"); graph.step(sg, feed, "none")
+            assert all(sum(p < 0 for p in win.table(s)) >= 6 for s in sg)          # pages behind the window are gone
+            pos = list(prefix)
+            outs = []
+            for piece in pieces:
+                feed = [s[p:p + n] for s, p, n in zip(full, pos, piece)]
+                a, b = eager.step(se, feed, "last"), graph.step(sg, feed, "last")
+                pos = [p + n for p, n in zip(pos, piece)]
+                assert max_err(a, b) < 2e-2, (again, r, piece, max_err(a, b))
+                for i in range(len(prefix)):
+                    assert max_err(b[i], refs[i][pos[i] - 1]) < tol("bfloat16", refs[i]), (again, r, piece, i)
+                outs.append(b.clone())
+            if again == 1:
+                recorded[r] = outs
+            elif again == 2:
+                assert all(torch.equal(x, y) for x, y in zip(recorded[r], outs)), r
+            eager.close(se); graph.close(sg)
+            graph.cache.check_consistent()
+    keys = set(graph._prompt_graphs)
+    assert all(k[2] == 1024 for k in keys) and {(1, 16, 1024, True), (1, 256, 1024, False), (1, 64, 1024, False),
+                                                (2, 16, 1024, False), (2, 144, 1024, True), (3, 80, 1024, True)} <= keys
+    assert all(g.graph is not None for g in graph._prompt_graphs.values())
+
+
 @pytest.mark.parametrize("name,dtype", [("tiny-c", "bfloat16"), ("tiny-b", "float32"), ("tiny-a", "bfloat16")])
 def test_captured_prompt_steps_match_eager_and_plain_on_every_replay(name, dtype, monkeypatch):
     """Steps of a few short prompts, or pieces of prompts, are recorded into HIP graphs as well (their token count
