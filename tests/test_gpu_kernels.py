@@ -686,8 +686,9 @@ def test_embed_from_fragment_layout():
 
 
 # ------------------------------------------------------------------ matrix-core attention over the fragment cache layout
-def frag_case(nH, nKV, d, lens, new, cap, window, seed, crafted=None):
-    """Like attention_case, with the cache filled by rope_cache_write in the fragment layout (no rotation)."""
+def frag_case(nH, nKV, d, lens, new, cap, window, seed, crafted=None, dense=False):
+    """Like attention_case, with the cache filled by rope_cache_write in the fragment layout (no rotation).
+    dense: the reference through the plain implementation's masked matrix form on the GPU (long sequences)."""
     B = len(lens)
     kp, vp, bt = paged(max(lens), nKV, d, torch.bfloat16, B, seed)
     qs, refs = [], []
@@ -705,7 +706,10 @@ def frag_case(nH, nKV, d, lens, new, cap, window, seed, crafted=None):
         ops.rope_cache_write(qkv, torch.empty(L, nH * d, dtype=torch.bfloat16, device=DEV), kp, vp, None, None, pos,
                              torch.full((L,), b, dtype=torch.int32, device=DEV), bt, num_heads=nH, num_kv_heads=nKV,
                              head_dim=d, rotary_dim=0, max_position=L - 1, kv_layout=ops.KV_FRAGMENT)
-        refs.append(P.attention_core(q.double(), k.double(), v.double(), scale, cap, window)[L - n:])
+        if dense:
+            refs.append(P.attention_dense(q.double().to(DEV), k.double().to(DEV), v.double().to(DEV), scale, cap, window)[L - n:].cpu())
+        else:
+            refs.append(P.attention_core(q.double(), k.double(), v.double(), scale, cap, window)[L - n:])
         qs.append(q[L - n:])
     q = torch.cat(qs).reshape(-1, nH * d).to(DEV)
     cu = [0]
@@ -878,6 +882,25 @@ def test_attention_mfma_prompts(nH, nKV, d, cap, window):
                                       max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant,
                                       out_layout=ops.LAYOUT_FRAG16)
                 assert torch.equal(acts_from_fragments(flat, T, nH * d), out.cpu())
+
+
+@pytest.mark.parametrize("nH,nKV,d", [(8, 4, 256), (32, 16, 128), (6, 2, 64), (8, 8, 128), (3, 3, 128)])   # (3, 3): see below
+@pytest.mark.parametrize("cap,window", [(50.0, None), (4.0, 1000)])
+def test_attention_mfma_prompts_that_make_more_blocks_than_cus(nH, nKV, d, cap, window):
+    """Long prompts: the kernels whose waves share keys through LDS then have more blocks than the chip has CUs and
+    deal the kv heads to the XCDs (blocks that read the same keys meet in one L2); with 1, 2, 4, 8 and 16 kv heads
+    times passes, and 6, a number that fits neither way (dealt plainly); whole prompts and a prompt on a cached prefix."""
+    cases = [((1300, 1100), (1300, 1100)), ((2500,), (1200,))]
+    if nKV == 3:
+        cases = [((2304, 2304), (2304, 2304))]       # 288 blocks of the one or two kv-head passes of (4, 1) and (4, 2) heads
+        nH, nKV = 4, 1 if cap == 4.0 else 2
+    for lens, new in cases:
+        q, kp, vp, bt, cu, ctx, ref, scale = frag_case(nH, nKV, d, lens, new, cap, window, seed=4, dense=True)
+        for variant in (ops.PREFILL_SHARED4, ops.PREFILL_SHARED8, ops.PREFILL_SHARED4X2, ops.PREFILL_AUTO):
+            out = torch.full_like(q, float("nan"))
+            ops.attention_prefill(q, kp, vp, out, cu, ctx, bt, num_heads=nH, n_seqs=len(lens), max_new=max(new),
+                                  max_context=max(lens), scale=scale, softcap=cap, window=window, variant=variant)
+            close(out, ref, 2e-2)
 
 
 @pytest.mark.parametrize("nH,nKV,d", FRAG_SHAPES)
