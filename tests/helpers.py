@@ -118,3 +118,15 @@ TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 
 def max_err(a: torch.Tensor, b: torch.Tensor) -> float:
     return (a.double().cpu() - b.double().cpu()).abs().max().item()
+
+
+def model_from_tensors(cfg, tensors, dtype):
+    """A model of the package filled with given tensors (by name, on the device), as the loader fills it from a folder."""
+    from alice_llm_amd.api import Model
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.parts import Precision
+    lm = CausalLM(cfg.plan(), Precision.of(dtype), tensors["model.norm.weight"].device)
+    for name in lm.param_specs():
+        lm.assign(name, tensors[name])
+    lm.finalize()
+    return Model(cfg, lm)

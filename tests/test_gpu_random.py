@@ -2,7 +2,8 @@
 engine in both dtypes against the plain implementation.  Every case draws head size, heads and groups, widths,
 vocabulary, number of layers, caps, window, eps and scale, then a batch of unequal prompts (sometimes in two
 pieces), some decode steps, and runs it twice so that the second run finds used slots and pages.  A second set of
-cases has the widths of real models and batches of up to 70 sequences, bfloat16 against the 32-bit path."""
+cases has the widths of real models and batches of up to 70 sequences: the 32-bit path against the plain
+implementation, and bfloat16 against the 32-bit path."""
 import os
 import random
 import tempfile
@@ -11,7 +12,7 @@ import pytest
 import torch
 
 import alice_llm_amd as alice
-from helpers import TOL, max_err, plain_model, random_tokens
+from helpers import TOL, max_err, model_from_tensors, plain_model, random_tokens
 
 pytestmark = pytest.mark.gpu
 _TMP = tempfile.TemporaryDirectory(prefix="alice_random_")
@@ -79,9 +80,12 @@ def test_random_widths_of_real_models_in_batches_up_to_70(case):
     """Widths, head counts and feed-forward widths as real models have them (one or two layers, a small vocabulary),
     batches of 1 to 70 unequal prompts in one or two pieces, then single tokens through captured steps or eagerly,
     their ids from the host or on the device: this is where the rules that pick kernels and tiles by size take their
-    branches.  The bfloat16 path against the 32-bit path on the same weights, every sequence alone and whole (the 32-bit
-    path at these widths is compared with the plain implementation in test_gpu_shapes.py).  The largest error stays
-    below 8 % of the logits' rms (4 to 5.5 % over 900 such cases); a k-tile or a head left out is far above that."""
+    branches.  Two comparisons.  The 32-bit path, every sequence alone and whole, against the plain implementation
+    (float64 on the GPU, the same tensors) on up to 20 of the sequences; and the bfloat16 path in the batch against
+    that 32-bit path on all of them: for the sequences past the twentieth the engine is its own reference, which a
+    mistake common to both paths would pass (they are covered by the first twenty, which take the same code with
+    other lengths).  The largest bfloat16 error stays below 8 % of the logits' rms (4 to 5.5 % over 900 such cases);
+    a k-tile or a head left out is far above that."""
     number = int(case.split("-")[1])
     rng = random.Random(case)
     d = rng.choice([64, 128, 256])
@@ -105,7 +109,12 @@ def test_random_widths_of_real_models_in_batches_up_to_70(case):
     lens = [rng.randint(1, rng.choice([20, 150, 400])) for _ in range(n_seq)]
     decode = rng.choice([1, 3, 12])
     seqs = [random_tokens(V, n + decode, 100 * number + i) for i, n in enumerate(lens)]
-    exact = alice.Model.random(cfg, seed=number, dtype="float32")
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.weights.loader import random_tensors
+    from plain.gemma2_plain import PlainGemma2
+    dev = torch.device("cuda", torch.cuda.current_device())
+    tensors = dict(random_tensors(CausalLM(cfg.plan(), "float32", "cpu").param_specs(), number, torch.bfloat16, dev))
+    exact = model_from_tensors(cfg, tensors, "float32")
     eng = exact.engine(max_tokens=1024, max_seqs=1, use_graphs=False)
     refs = []
     for s in seqs:
@@ -113,8 +122,14 @@ def test_random_widths_of_real_models_in_batches_up_to_70(case):
         refs.append(eng.step(slot, [s], "all").cpu())
         eng.close(slot)
     del eng, exact
+    plain = PlainGemma2(raw, tensors, dense=True, device=dev)
+    for s, r in list(zip(seqs, refs))[:20]:
+        want = plain.forward(s).float().cpu()
+        assert max_err(r, want) < TOL["float32"] * max(1.0, float(want.abs().max())), (raw, len(s), max_err(r, want))
+    del plain
+    torch.cuda.empty_cache()
     rms = min(float(r.pow(2).mean().sqrt()) for r in refs)
-    model = alice.Model.random(cfg, seed=number, dtype="bfloat16")
+    model = model_from_tensors(cfg, tensors, "bfloat16")
     eng = model.engine(seq_lens=[len(s) for s in seqs], max_seqs=n_seq, use_graphs=rng.random() < 0.7)
     for again in range(2):
         slots = eng.open(n_seq)

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import alice_llm_amd as alice
-from helpers import TOL, max_err, plain_model, random_tokens
+from helpers import model_from_tensors, TOL, max_err, plain_model, random_tokens
 
 pytestmark = pytest.mark.gpu
 
@@ -109,18 +109,6 @@ def test_odd_sizes_whole_and_token_by_token(name):
         assert max_err(torch.cat(cut), ref) < TOL[dtype] * scale, (dtype, max_err(torch.cat(cut), ref))
 
 
-def _model_from_tensors(cfg, tensors, dtype):
-    """A model of the package filled with given tensors (by name, on the device), as the loader fills it from a folder."""
-    from alice_llm_amd.api import Model
-    from alice_llm_amd.engine.model import CausalLM
-    from alice_llm_amd.parts import Precision
-    lm = CausalLM(cfg.plan(), Precision.of(dtype), tensors["model.norm.weight"].device)
-    for name in lm.param_specs():
-        lm.assign(name, tensors[name])
-    lm.finalize()
-    return Model(cfg, lm)
-
-
 def test_full_2b_shape_against_the_plain_implementation():
     """The whole Gemma 2 2B shape (26 layers, vocabulary 256,000) with random weights: a prompt and 8 single tokens,
     the 32-bit path and the bfloat16 path against the plain implementation, which runs in float64 on the GPU on the
@@ -170,7 +158,7 @@ def test_full_2b_shape_against_the_plain_implementation():
         torch.cuda.empty_cache()
         assert ref.shape == (n_tokens, 256000) and 0.5 < float(ref.pow(2).mean().sqrt()) < 2.0 and float(ref.abs().max()) > 4.0
         for dtype in ("float32", "bfloat16") if variant == "as drawn" else ("float32",):
-            model = _model_from_tensors(cfg, tensors, dtype)
+            model = model_from_tensors(cfg, tensors, dtype)
             eng = model.engine(seq_lens=[320], max_seqs=1)
             s = eng.open(1)
             got = [eng.step(s, [toks[:-8]], "all")] + [eng.step(s, [[t]], "last").clone() for t in toks[-8:]]
