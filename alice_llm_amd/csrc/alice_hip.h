@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 5
+#define ALICE_ABI_VERSION 6
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
@@ -79,10 +79,13 @@ int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, i
                             const int* seq_of_token, const int* block_table, int bt_stride, int nH, int nKV, int d,
                             int page_size, int n_pages, int kv_layout, hipStream_t stream);
 
+// bias_slopes: null, or nH floats: head h's capped score of key k for the query at position p gets
+// bias_slopes[h] * (k - p) added before the softmax (a linear distance bias at the score stage).
 int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
                             const int* positions, const int* seq_of_token, const int* block_table,
                             int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
-                            float softcap, int window, int full_precision, hipStream_t stream);
+                            float softcap, int window, const float* bias_slopes, int full_precision,
+                            hipStream_t stream);
 
 // bfloat16 attention on the matrix cores over a cache in the fragment layout (kv_layout 1 of
 // alice_rope_cache_write): prompts, and single tokens with the keys split over `splits` blocks.

@@ -6,7 +6,10 @@
 // cap * tanh(s / cap), then the softmax over the keys max(0, pos + 1 - window) .. pos (window keys,
 // the query's own included, llama3.rs:5444-5451), then the weighted sum of the values; the kv head
 // of query head h is h / (nH / nKV).  The softmax is computed chunk by chunk with a running maximum
-// (the reference's online variant, llama3.rs:5568-5620).
+// (the reference's online variant, llama3.rs:5568-5620).  A position term at the score stage is a
+// parameter: with bias_slopes, head h's capped score of key k for the query at position p gets
+// bias_slopes[h] * (k - p) added (a linear distance bias; the reference's models have none, so the
+// product passes a null pointer).
 #include "common.h"
 #include "alice_hip.h"
 
@@ -20,7 +23,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pool, const T* __restrict__ v_pool, T* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int bt_stride, int nH, int nKV, int d, int page_size,
-    float scale, float cap, int window, int DG) {
+    float scale, float cap, int window, int DG, const float* __restrict__ bias_slopes) {
   __shared__ float qs[256];
   __shared__ float sc[CHUNK];
   __shared__ float red[17];
@@ -30,6 +33,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
   const int pos = positions[t];
   const int seq = seq_of_token[t];
   const int kvh = h / (nH / nKV);
+  const float slope = bias_slopes ? bias_slopes[h] : 0.f;
   const int start = window > 0 ? max(0, pos + 1 - window) : 0;
   const int* bt = block_table + (size_t)seq * bt_stride;
 
@@ -52,6 +56,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
       for (int e = 0; e < d; ++e) s = fmaf(qs[e], load_f32(krow, e), s);
       s *= scale;
       if (cap > 0.f) s = cap * (FULL ? tanh_full(s / cap) : tanh_fast(s / cap));
+      if (bias_slopes) s = fmaf(slope, (float)(kp - pos), s);
       sc[i] = s;
       lmax = fmaxf(lmax, s);
     }
@@ -90,7 +95,8 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
 extern "C" int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
                                        const int* positions, const int* seq_of_token, const int* block_table,
                                        int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
-                                       float softcap, int window, int full_precision, hipStream_t stream) {
+                                       float softcap, int window, const float* bias_slopes, int full_precision,
+                                       hipStream_t stream) {
   ALICE_CHECK(dtype_ok(dtype), "attention: unknown dtype %d", dtype);
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
   ALICE_CHECK(d >= 1 && d <= 256, "attention: head_dim %d is outside 1..256, the range of this kernel", d);
@@ -104,10 +110,10 @@ extern "C" int alice_attention_generic(const void* q, int dtype, const void* k_p
   DISPATCH_DTYPE(dtype, TT, {
     if (full_precision)
       attn_generic_kernel<TT, true><<<grid, THREADS, 0, stream>>>((const TT*)q, (const TT*)k_pool, (const TT*)v_pool,
-          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG);
+          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes);
     else
       attn_generic_kernel<TT, false><<<grid, THREADS, 0, stream>>>((const TT*)q, (const TT*)k_pool, (const TT*)v_pool,
-          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG);
+          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes);
   });
   ALICE_LAUNCH_CHECK();
   return 0;

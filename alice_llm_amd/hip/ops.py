@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib = None
 _lib_path = None
@@ -48,7 +48,7 @@ def _declare(lib) -> None:
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
-        "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, P],
+        "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -382,7 +382,9 @@ def linear_rope_cache(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, k_p
 def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor,
                       positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, *,
                       num_heads: int, scale: float, softcap: Optional[float], window: Optional[int],
-                      max_position: int, full_precision: bool) -> None:
+                      max_position: int, full_precision: bool, bias_slopes: Optional[torch.Tensor] = None) -> None:
+    """bias_slopes: float32 [num_heads]; head h's capped score of key k for the query at position p gets
+    bias_slopes[h] * (k - p) added before the softmax."""
     T = q.shape[0]
     dt = q.dtype
     if k_pool.dim() != 4:
@@ -397,10 +399,13 @@ def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
     _dev(block_table, "block_table", torch.int32)
     if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
         raise HipLibraryError(f"position {max_position} is beyond the block table {tuple(block_table.shape)}")
+    if bias_slopes is not None:
+        _dev(bias_slopes, "bias_slopes", torch.float32, (num_heads,))
     _call("alice_attention_generic", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), v_pool.data_ptr(),
           out.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], T, num_heads, nKV, d, page_size, float(scale),
-          float(softcap or 0.0), int(window or 0), int(full_precision), _stream())
+          float(softcap or 0.0), int(window or 0), None if bias_slopes is None else bias_slopes.data_ptr(),
+          int(full_precision), _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
@@ -530,11 +535,14 @@ def linear_parts(parts: torch.Tensor, splits: int, w: torch.Tensor, y: torch.Ten
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,
               block_table: torch.Tensor, *, num_heads: int, scale: float, softcap: Optional[float],
               window: Optional[int], full_precision: bool, kv_layout: int = KV_ROW,
-              out_layout: int = LAYOUT_ROW) -> None:
+              out_layout: int = LAYOUT_ROW, bias_slopes: Optional[torch.Tensor] = None) -> None:
     """Attention of the step's query tokens over the cache; picks the kernel for the step's shape and
     the cache's layout.  `ctx` carries positions, seq_of_token, cu_seqlens, context_lens and the
-    host-side sizes of the step.  out_layout FRAG16 is taken by the matrix-core kernels only."""
+    host-side sizes of the step.  out_layout FRAG16 is taken by the matrix-core kernels only; a score bias
+    (bias_slopes, see attention_generic) by the generic kernel only, over a row-major cache."""
     if kv_layout == KV_FRAGMENT:
+        if bias_slopes is not None:
+            raise HipLibraryError("the matrix-core attention kernels take no score bias: lay the cache out row-major")
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
             attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
@@ -550,7 +558,7 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
         raise HipLibraryError("only the matrix-core attention kernels write fragment order")
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
-                      max_position=ctx.max_position, full_precision=full_precision)
+                      max_position=ctx.max_position, full_precision=full_precision, bias_slopes=bias_slopes)
 
 
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -5,11 +5,14 @@ head h with kv head h // (nH // nKV): score = (q . k) * scale, softcap cap * tan
 softmax over the keys max(0, pos + 1 - window) .. pos, weighted sum of v, output projection
 (llama3.rs:14206-14217, 14307-14331, 5431-5451, 5622-5688, 14423).  Scale, softcap, window, head
 counts and head size are constructor arguments; window None is global attention, softcap None
-turns the tanh off.
+turns the tanh off.  A position term at the score stage is a constructor argument too:
+score_bias_slopes, one slope a query head, adds slope * (key position - query position) to the
+capped score (a linear distance bias; the 32-bit attention kernel over a row-major cache takes it,
+in both dtypes).
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict, Optional, Sequence
 
 import torch
 
@@ -24,7 +27,8 @@ class Attention(Part):
 
     def __init__(self, precision: Precision, positions: dict, *, hidden_size: int, num_heads: int,
                  num_kv_heads: int, head_dim: int, scale: float, softcap: Optional[float] = None,
-                 window: Optional[int] = None, position: Optional[str] = None):
+                 window: Optional[int] = None, position: Optional[str] = None,
+                 score_bias_slopes: Optional[Sequence[float]] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
         if not 1 <= head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
@@ -36,6 +40,10 @@ class Attention(Part):
         self.scale = float(scale)
         self.softcap = None if softcap is None else float(softcap)
         self.window = window
+        if score_bias_slopes is not None and len(score_bias_slopes) != num_heads:
+            raise ValueError(f"attention: {len(score_bias_slopes)} score bias slopes for {num_heads} heads")
+        self.score_bias_slopes = None if score_bias_slopes is None else [float(v) for v in score_bias_slopes]
+        self._slopes: Optional[torch.Tensor] = None
         self.position = positions[position] if position is not None else positions.get("none")
         if self.position is None:
             raise ValueError("attention needs a position encoding (use 'none' for no rotation)")
@@ -46,7 +54,8 @@ class Attention(Part):
         # layout; every other case is row-major.  It depends on the arithmetic and the head size alone, so
         # that a run that reads another run's cache finds the layout it expects.
         self.kv_layout = (ops.KV_FRAGMENT if precision.name == "bfloat16" and precision.act == torch.bfloat16
-                          and ops.library_ready() and ops.attention_mfma_supported(head_dim) else ops.KV_ROW)
+                          and ops.library_ready() and ops.attention_mfma_supported(head_dim)
+                          and score_bias_slopes is None else ops.KV_ROW)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -80,6 +89,8 @@ class Attention(Part):
         if self.pair_order:
             w = w[order.to(w.device)]
         self.qkv.load(w)
+        if self.score_bias_slopes is not None:
+            self._slopes = torch.tensor(self.score_bias_slopes, dtype=torch.float32, device=w.device)
 
     def weight_bytes(self) -> int:
         return self.qkv.nbytes() + self.o.nbytes()
@@ -120,5 +131,6 @@ class Attention(Part):
         out = FragmentActs.empty(T, self.q_dim, q.device) if frag else torch.empty_like(q)
         ops.attention(q, cache.k, cache.v, out.data if frag else out, ctx, cache.block_table, num_heads=self.nH,
                       scale=self.scale, softcap=self.softcap, window=self.window, full_precision=self.precision.full,
-                      kv_layout=self.kv_layout, out_layout=ops.LAYOUT_FRAG16 if frag else ops.LAYOUT_ROW)
+                      kv_layout=self.kv_layout, out_layout=ops.LAYOUT_FRAG16 if frag else ops.LAYOUT_ROW,
+                      bias_slopes=self._slopes)
         return self.o(out, torch.float32, allow_partials=True)

@@ -125,7 +125,7 @@ def model_from_tensors(cfg, tensors, dtype):
     from alice_llm_amd.api import Model
     from alice_llm_amd.engine.model import CausalLM
     from alice_llm_amd.parts import Precision
-    lm = CausalLM(cfg.plan(), Precision.of(dtype), tensors["model.norm.weight"].device)
+    lm = CausalLM(cfg.plan(), Precision.of(dtype), next(iter(tensors.values())).device)
     for name in lm.param_specs():
         lm.assign(name, tensors[name])
     lm.finalize()

@@ -279,6 +279,57 @@ def test_attention_far_key_and_window_edge(dt):
         assert (abs(float(out[0, 0]) - 7.0) < 1e-2) == seen
 
 
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cap,window", [(None, None), (5.0, 40)])
+def test_attention_generic_with_a_distance_bias_at_the_score_stage(dt, cap, window):
+    """A position term at the score stage as a parameter of the kernel: head h's capped score of key k for the
+    query at position p gets slope[h] * (k - p) added.  Against a dense reference written here (the plain
+    implementation of the product's architecture has no such term): prompts on a cached prefix and single tokens.
+    Slopes of zero give the bits of the call without slopes, and a steep slope leaves every query its own value."""
+    nH, nKV, d = 6, 2, 24
+    slopes = torch.tensor([0.0, 0.5, 0.25, 0.125, 0.0625, 0.03125], dtype=D)
+    for lens, new in (((70, 131), (70, 9)), ((150, 3, 65), (1, 1, 1))):
+        B = len(lens)
+        kp, vp, bt = paged(max(lens), nKV, d, DT[dt], B, 8)
+        scale = 1.0 / math.sqrt(d)
+        qs, refs, pos, seq = [], [], [], []
+        for b, (L, n) in enumerate(zip(lens, new)):
+            g = torch.Generator().manual_seed(800 + b)
+            q, k, v = (torch.randn(L, h, d, generator=g, dtype=D).to(DT[dt]).double() for h in (nH, nKV, nKV))
+            fill_pools(kp, vp, bt, k, v, b)
+            ar = torch.arange(L)
+            dist = (ar[None, :] - ar[:, None]).double()                         # key position - query position
+            out = torch.empty(L, nH, d, dtype=D)
+            for h in range(nH):
+                sc = (q[:, h] @ k[:, h // (nH // nKV)].T) * scale
+                if cap is not None:
+                    sc = cap * torch.tanh(sc / cap)
+                sc = sc + slopes[h] * dist
+                seen = (dist <= 0) & ((dist > -window) if window else torch.ones_like(dist, dtype=torch.bool))
+                out[:, h] = torch.softmax(sc.masked_fill(~seen, float("-inf")), dim=-1) @ v[:, h // (nH // nKV)]
+            refs.append(out[L - n:])
+            qs.append(q[L - n:])
+            pos += list(range(L - n, L))
+            seq += [b] * n
+        q = torch.cat(qs).reshape(-1, nH * d).to(DT[dt]).to(DEV)
+        pos_t, seq_t = (torch.tensor(a, dtype=torch.int32, device=DEV) for a in (pos, seq))
+        ref = torch.cat(refs).reshape(-1, nH * d)
+        kw = dict(num_heads=nH, scale=scale, softcap=cap, window=window, max_position=max(lens) - 1, full_precision=dt == "float32")
+        out = torch.empty_like(q)
+        ops.attention_generic(q, kp, vp, out, pos_t, seq_t, bt, bias_slopes=slopes.float().to(DEV), **kw)
+        close(out, ref, 2e-5 if dt == "float32" else 2e-2)
+        plain, zero = torch.empty_like(q), torch.empty_like(q)
+        ops.attention_generic(q, kp, vp, plain, pos_t, seq_t, bt, **kw)
+        ops.attention_generic(q, kp, vp, zero, pos_t, seq_t, bt, bias_slopes=torch.zeros(nH, device=DEV), **kw)
+        assert torch.equal(plain, zero) and (plain.float() - out.float()).abs().max() > 0.05
+        steep = torch.empty_like(q)
+        ops.attention_generic(q, kp, vp, steep, pos_t, seq_t, bt, bias_slopes=torch.full((nH,), 200.0, device=DEV), **kw)
+        own = torch.stack([vp[int(bt[b, p // 64]), :, p % 64] for b, p in zip(seq, pos)]).float()          # [T, nKV, d]
+        assert (steep.view(-1, nKV, nH // nKV, d).float() - own[:, :, None]).abs().max() < 1e-5
+    with pytest.raises(ops.HipLibraryError, match="bias_slopes"):
+        ops.attention_generic(q, kp, vp, out, pos_t, seq_t, bt, bias_slopes=torch.zeros(nH + 1, device=DEV), **kw)
+
+
 def test_attention_refuses_sizes_it_does_not_cover():
     q, kp, vp, bt, pos, seq, ref, scale = attention_case("float32", 2, 1, 16, (9,), (9,), None, None, seed=6)
     out = torch.empty_like(q)

@@ -13,6 +13,7 @@ from alice_llm_amd.cache import Cache
 from alice_llm_amd.config.plan import LayerPlan, ModelPlan, PartSpec, ScheduleEntry
 from alice_llm_amd.engine.model import CausalLM
 from alice_llm_amd.engine.step import Engine
+from alice_llm_amd.hip import ops
 from alice_llm_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, CacheNeed, ParamSpec, Part, Precision,
                                  ResidualStream, StateNeed)
 from alice_llm_amd.weights.loader import init_random
@@ -835,6 +836,112 @@ def test_toy_architecture_with_routing_and_another_position_encoding():
     assert (cut - whole).abs().max() < 1e-5
     eng.cache.check_consistent()
 
+
+class ToyDistanceBiasConfig(ToyConfig):
+    """Positions known to the scores alone: attention without rotation whose heads subtract slope * distance (one
+    slope a head, a constructor argument of the attention mixer), global and windowed layers in turn."""
+    SLOPES = (0.5, 0.125, 0.03125, 0.0)
+
+    def plan(self):
+        H, V = self.d["width"], self.d["vocab"]
+        norm = lambda name: PartSpec("rmsnorm", {"dim": H, "eps": 1e-5, "weight_offset": 0.0}, name)
+        att = lambda i: PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": self.d["head"],
+                                               "scale": 0.2, "softcap": 4.0 if i % 2 else None, "window": 6 if i % 2 else None,
+                                               "position": "none", "score_bias_slopes": self.SLOPES}, "attn")
+        layers = [LayerPlan(block="prenorm", mixer=att(i), feed_forward=PartSpec("toy_graph_mlp", {"hidden_size": H}, "ff"),
+                            norms={"pre_mixer": norm("n1"), "pre_ff": norm("n2")}, prefix=f"blocks.{i}.") for i in range(self.d["depth"])]
+        return ModelPlan(vocab_size=V, hidden_size=H, max_positions=128,
+                         embedding=PartSpec("embedding", {"vocab_size": V, "dim": H, "scale": 1.0}, "emb"), positions={},
+                         layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in range(self.d["depth"])),
+                         final_norm=norm("final"), head=PartSpec("lm_head", {"vocab_size": V, "dim": H, "tied_to": "emb"}, "head"))
+
+
+def toy_distance_bias_plain(raw, tensors, tokens):
+    """Whole sequence in 64-bit from the stored tensors (by name), dense attention with the distance term."""
+    H, d = raw["width"], raw["head"]
+    w = lambda name: tensors[name].double().cpu()
+    E = w("emb.weight")
+    x = E[torch.tensor(tokens)]
+    T = len(tokens)
+    rms = lambda v, g: v * torch.rsqrt((v * v).mean(-1, keepdim=True) + 1e-5) * g
+    ar = torch.arange(T)
+    dist = (ar[None, :] - ar[:, None]).double()
+    for i in range(raw["depth"]):
+        pre = f"blocks.{i}."
+        h = rms(x, w(pre + "n1.weight"))
+        q, k, v = ((h @ w(pre + f"attn.{n}_proj.weight").T).view(T, -1, d) for n in "qkv")
+        cap, window = (4.0, 6) if i % 2 else (None, None)
+        heads = []
+        for hd in range(4):
+            sc = (q[:, hd] @ k[:, hd // 2].T) * 0.2
+            if cap:
+                sc = cap * torch.tanh(sc / cap)
+            sc = sc + ToyDistanceBiasConfig.SLOPES[hd] * dist
+            seen = (dist <= 0) & ((dist > -window) if window else (dist <= 0))
+            heads.append(torch.softmax(sc.masked_fill(~seen, float("-inf")), -1) @ v[:, hd // 2])
+        x = x + torch.stack(heads, 1).reshape(T, 4 * d) @ w(pre + "attn.o_proj.weight").T
+        h = rms(x, w(pre + "n2.weight"))
+        x = x + torch.relu(h @ w(pre + "ff.w.weight").T)
+    return rms(x, w("final.weight")) @ E.T
+
+
+@pytest.mark.parametrize("dtype,head", [("float32", 16), ("bfloat16", 16), ("bfloat16", 64)])
+def test_toy_architecture_with_a_position_term_at_the_score_stage(dtype, head):
+    """Another kind of position encoding, registered from here: no rotation, a distance term in the scores.  It is a
+    parameter of the attention mixer (score_bias_slopes), so the toy needs no mixer and no kernel of its own; with
+    it the mixer keeps its cache row-major and takes the 32-bit attention kernel, also where the head size (64)
+    would otherwise go to the matrix cores.  Whole prompts, then single tokens through captured steps, against a
+    64-bit replica that reads the stored tensors; without the term the logits differ by far more than the bound."""
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.weights.loader import random_tensors
+    from helpers import model_from_tensors
+    FEED_FORWARDS.register("toy_graph_mlp", ToyGraphMLP)
+    alice.register_architecture("ToyDistanceBiasForCausalLM", ToyDistanceBiasConfig)
+    raw = {"architectures": ["ToyDistanceBiasForCausalLM"], "width": 64, "vocab": 83, "depth": 3, "head": head}
+    cfg = alice.config_from_dict(raw)
+    stored = torch.float32 if dtype == "float32" else torch.bfloat16
+    tensors = dict(random_tensors(CausalLM(cfg.plan(), "float32", "cpu").param_specs(), 9, stored, DEV))
+    for k in tensors:                                           # norm weights about 1 and matrices of 0.12: logits and scores of order 1
+        if "proj.weight" in k or k == "emb.weight":
+            tensors[k] = (tensors[k].float() * 6.0).to(stored)
+        elif k.endswith(("n1.weight", "n2.weight", "final.weight")):
+            tensors[k] = (tensors[k].float() + 1.0).to(stored)
+    model = model_from_tensors(cfg, tensors, dtype)
+    mixers = [l.mixer for l in model.lm.layers]
+    assert all(m.kv_layout == ops.KV_ROW and m._slopes is not None for m in mixers)
+    seqs = [[5, 9, 3, 60, 1, 22, 8, 8, 41, 2, 13, 0, 33, 17, 70, 4, 4, 29], [7, 7, 30, 12, 55, 81, 2]]
+    refs = [toy_distance_bias_plain(raw, tensors, t) for t in seqs]
+    assert max(float(r.abs().max()) for r in refs) > 2.0
+    tol = (2e-5 if dtype == "float32" else 4e-2) * max(1.0, max(float(r.abs().max()) for r in refs))
+    eng = model.engine(max_tokens=256, max_seqs=2)
+    slots = eng.open(2)
+    whole = eng.step(slots, seqs, "all")
+    eng.close(slots)
+    assert (whole.double().cpu() - torch.cat(refs)).abs().max() < tol
+    for again in range(3):                                      # the third pass replays captured single-token steps
+        slots = eng.open(2)
+        got = {0: [], 1: []}
+        first = eng.step(slots, [s[:4] for s in seqs], "last")
+        for i in range(4, len(seqs[0])):
+            live = [b for b in (0, 1) if i < len(seqs[b])]
+            lg = eng.step([slots[b] for b in live], [[seqs[b][i]] for b in live], "last")
+            for row, b in enumerate(live):
+                got[b].append(lg[row].clone())
+            if i + 1 == len(seqs[1]):
+                eng.close([slots[1]])
+        eng.close([slots[0]])
+        for b in (0, 1):
+            assert (first[b].double().cpu() - refs[b][3]).abs().max() < tol
+            assert (torch.stack(got[b]).double().cpu() - refs[b][4:]).abs().max() < tol, (again, b)
+    assert eng.use_graphs and len(eng._graphs) >= 1
+    # the term matters: the same tensors without it are far from the replica
+    for m in mixers:
+        m._slopes = None
+    slots = eng.open(2)
+    flat = eng.step(slots, seqs, "all")
+    eng.close(slots)
+    assert (flat.double().cpu() - torch.cat(refs)).abs().max() > 10 * tol
+    eng.cache.check_consistent()
 
 
 @pytest.mark.parametrize("prec", PRECS)
